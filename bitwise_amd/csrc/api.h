@@ -86,4 +86,36 @@ int bw_chain_end(void* stream);
 int bw_sample(const float* logits, int vocab, int ld, int rows, const float* temperature, const double* uniform,
               int32_t* out, void* stream);
 int bw_fingerprint(const float* logits, int vocab, int ld, int rows, const void* h_in, void* h_out, void* stream);
+// Mixers with a fixed-size state per request (sequence_mix.hip).  seq_rows: [requests, 2] = (first row, rows) of every
+// request of the step; slots: its state slot.  A request without rows, with a negative slot or a negative first
+// position is padding: its state stays as it is.
+int bw_norm_shift(const float* x, int ldx, const float* w, const float* mix, float* state, long long state_ld,
+                  const int32_t* positions, const int32_t* row_seq, const int32_t* seq_rows, const int32_t* slots,
+                  void* out, int out_is_bf16, int ldo, int rows, int dim, float eps, void* stream);
+// mode 0: a decay per key channel (gate: logits [rows, ldg] at gate_off, bias [heads*dim], param = 1/tau);
+// mode 1: scalar input and forget gates per head (columns gate_off and gate2_off of proj, biases bias and bias2, param = cap)
+// with normaliser and running maximum.  state: [slots, state_ld] of S [heads][dim][vdim] (mode 1: then n [heads][dim], m [heads]).
+int bw_linear_recurrence(int mode, const float* proj, int ldp, int q_off, int k_off, int v_off, const float* gate, int ldg,
+                         int gate_off, int gate2_off, const float* bias, const float* bias2, float param, float qscale,
+                         float* state, long long state_ld, float* out, int ldo, const int32_t* seq_rows,
+                         const int32_t* slots, const int32_t* positions, int nseq, int heads, int dim, int vdim,
+                         void* stream);
+// gate 0: sigmoid, 1: SiLU.  weight: [heads, wstride] (wstride 0: one weight vector for all heads).
+int bw_head_norm_gate(const float* o, int ldi, const float* weight, int wstride, const float* g, int ldg, int gate, void* out,
+                      int out_is_bf16, int ldo, const int32_t* positions, int rows, int heads, int vdim, float eps,
+                      void* stream);
+// h = act(gate) * up of the stacked 32-bit product [rows, 2*inter]; act 0: SiLU, 1: GELU in its tanh form.
+int bw_glu(const float* gate_up, void* h, int out_is_bf16, int rows, int inter, int act, void* stream);
+// Attention over a compressed cache shared by all heads (latent_attention.hip).
+int bw_latent_prep(const float* proj, int ldp, int q_off, int dkv_off, const float* norm_w, float eps,
+                   const float* cos_table, const float* sin_table, const int32_t* positions, const int32_t* row_seq,
+                   const int32_t* block_table, int table_stride, void* cache, int cache_is_bf16, float* qa, int ldqa,
+                   int rows, int heads, int dim, int rot, int rotary, int rank, int page_size, int write_cache,
+                   void* stream);
+int bw_headwise_linear(const float* x, int ldx, int xhs, const void* wt, int w_is_bf16, int in, int outn, void* out,
+                       int out_is_bf16, int ldo, int ohs, int rows, int heads, void* stream);
+int bw_shared_key_attention(const float* q, int ldq, const int32_t* positions, const int32_t* block_table,
+                            int table_stride, const int32_t* tiles, int num_tiles, const void* cache, int cache_is_bf16,
+                            int num_pages, const float* sink, float* out, int ldo, int heads, int dk, int dv,
+                            int page_size, int window, float scale, int heads_per_group, void* stream);
 }

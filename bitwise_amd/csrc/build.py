@@ -23,7 +23,7 @@ from typing import List, Optional
 
 HERE = Path(__file__).resolve().parent
 SOURCES = ["elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_f32.hip", "attention_bf16.hip",
-           "fused_decode.hip", "sampling.hip"]
+           "fused_decode.hip", "sampling.hip", "sequence_mix.hip", "latent_attention.hip"]
 HEADERS = ["common.h", "api.h", "layout.h", "gemm_bf16_skinny.h", "gemm_bf16_tiles.h", "gemm_bf16_rows.h",
            "gemm_bf16_phases.h"]
 LIB_NAME = "libbitwise_hip.so"
@@ -110,7 +110,7 @@ def build(force: bool = False, verbose: bool = True) -> Path:
             _say(f"compiled {name} ({time.time() - t0:.0f} s)")
         return str(obj)
 
-    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(compile_one, SOURCES))
     tmp_lib = out_dir / (LIB_NAME + f".tmp{os.getpid()}")
     # -z defs: a kernel template that the host pass failed to instantiate (it can do so without a

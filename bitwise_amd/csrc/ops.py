@@ -76,6 +76,21 @@ _SIGS = {
     "bw_chain_end": [c_void_p],
     "bw_sample": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_fingerprint": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "bw_norm_shift": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
+                      c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "bw_linear_recurrence": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
+                             c_float, c_float, c_void_p, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                             c_int, c_int, c_int, c_void_p],
+    "bw_head_norm_gate": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int,
+                          c_int, c_int, c_float, c_void_p],
+    "bw_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_latent_prep": [c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                       c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                       c_void_p],
+    "bw_headwise_linear": [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
+                           c_int, c_void_p],
+    "bw_shared_key_attention": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int,
+                                c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
 }
 
 _fns = {}
@@ -315,8 +330,10 @@ def rope_kvwrite(qkv: torch.Tensor, q_out: Optional[torch.Tensor], positions: to
 # ------------------------------------------------------------------------------ matrix products
 
 def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, accumulate: bool = False) -> None:
-    """out[:rows] (+)= x[:rows] @ w.T with one k-ascending fused multiply-add chain per output."""
-    _need(x, torch.float32, "x")
+    """out[:rows] (+)= x[:rows] @ w.T with one k-ascending fused multiply-add chain per output.  ``x`` may be a
+    column slice of a wider matrix (rows apart by its stride)."""
+    if not x.is_cuda or x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+        raise ValueError("gemm_f32: x must be a float32 GPU matrix with contiguous rows")
     _need(out, torch.float32, "out")
     if not w.is_cuda or not w.is_contiguous() or w.dim() != 2:
         raise ValueError("gemm_f32: weight must be a contiguous [N, K] GPU tensor")
@@ -627,6 +644,192 @@ def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor
                                         block_table.stride(0), cos.data_ptr(), sin.data_ptr(), k_cache.data_ptr(),
                                         v_cache.data_ptr(), rows, heads, kv_heads, head_dim, K, page_size,
                                         int(write_cache), _stream()), "gemm_qkv_rope_bf16")
+
+
+# ------------------------------------------------------------------------------ mixers with a state per request
+
+RECUR_DECAY_PER_CHANNEL, RECUR_SCALAR_GATES = 0, 1
+RECUR_MAX_DIM = 128          # key channels of a head that the recurrence keeps in a lane's registers
+GATE_SIGMOID, GATE_SILU = 0, 1
+ACT_SILU, ACT_GELU_TANH = 0, 1
+
+
+def _act_out(t: torch.Tensor, what: str) -> int:
+    if not t.is_cuda or not t.is_contiguous():
+        raise ValueError(f"{what} must be a contiguous GPU tensor")
+    return _is_bf16(t, what)
+
+
+def norm_shift(x: torch.Tensor, weight: torch.Tensor, mix: torch.Tensor, state: torch.Tensor, positions: torch.Tensor,
+               row_seq: torch.Tensor, seq_rows: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, rows: int,
+               eps: float) -> None:
+    """out[r] = h[r] + (h_prev[r] - h[r]) * mix with h = rmsnorm(x) * weight and h_prev the h of the request's token
+    before (from ``state`` [slots, width] for a request's first row of the step, which then receives the h of
+    the request's last row).  All 32-bit; ``out`` in float32 or bfloat16."""
+    _need(x, torch.float32, "x")
+    _need(weight, torch.float32, "norm weight")
+    _need(mix, torch.float32, "mix")
+    _need(state, torch.float32, "state")
+    for t, what in ((positions, "positions"), (row_seq, "row_seq"), (seq_rows, "seq_rows"), (slots, "slots")):
+        _need(t, torch.int32, what)
+    dim = x.shape[1]
+    if weight.numel() != dim or mix.numel() != dim or state.dim() != 2 or state.shape[1] < dim:
+        raise ValueError("norm_shift: weight, mix or state do not fit the rows' width")
+    if x.shape[0] < rows or out.shape[0] < rows or out.shape[1] != dim or positions.numel() < rows or row_seq.numel() < rows:
+        raise ValueError("norm_shift: buffers shorter than the rows")
+    _check(_fn("bw_norm_shift")(x.data_ptr(), x.stride(0), weight.data_ptr(), mix.data_ptr(), state.data_ptr(), state.stride(0),
+                                positions.data_ptr(), row_seq.data_ptr(), seq_rows.data_ptr(), slots.data_ptr(),
+                                out.data_ptr(), _act_out(out, "out"), out.stride(0), rows, dim, float(eps), _stream()),
+           "norm_shift")
+
+
+def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gate: torch.Tensor, gate_off: int,
+                      gate2_off: int, bias: torch.Tensor, bias2: Optional[torch.Tensor], param: float, qscale: float,
+                      state: torch.Tensor, out: torch.Tensor, seq_rows: torch.Tensor, slots: torch.Tensor,
+                      positions: torch.Tensor, nseq: int, heads: int, dim: int, vdim: int) -> None:
+    """The recurrence S <- decay * S + k v^T, o = S^T (q * qscale) per head over every request's rows in order, from and
+    to ``state`` [slots, elements].  RECUR_DECAY_PER_CHANNEL: decay = exp(logsigmoid(gate + bias) * param) per key
+    channel (``gate`` [rows, >= gate_off + heads*dim]).  RECUR_SCALAR_GATES: capped input and forget gates per head
+    (columns gate_off + h and gate2_off + h of ``gate``), a normaliser and a running maximum in the state; param = cap."""
+    _need(proj, torch.float32, "proj")
+    _need(gate, torch.float32, "gate")
+    _need(bias, torch.float32, "bias")
+    _need(state, torch.float32, "state")
+    _need(out, torch.float32, "out")
+    for t, what in ((positions, "positions"), (seq_rows, "seq_rows"), (slots, "slots")):
+        _need(t, torch.int32, what)
+    if dim > RECUR_MAX_DIM:
+        raise ValueError(f"linear_recurrence: {dim} key channels a head; the kernel keeps up to {RECUR_MAX_DIM}")
+    if mode == RECUR_SCALAR_GATES:
+        if bias2 is None:
+            raise ValueError("linear_recurrence: scalar gates need both biases")
+        _need(bias2, torch.float32, "bias2")
+        if bias.numel() != heads or bias2.numel() != heads or max(gate_off, gate2_off) + heads > gate.shape[1]:
+            raise ValueError("linear_recurrence: gates or biases do not fit the heads")
+        need = heads * (dim * vdim + dim + 1)
+    else:
+        if bias.numel() != heads * dim or gate_off + heads * dim > gate.shape[1]:
+            raise ValueError("linear_recurrence: decay logits or bias do not fit heads x dim")
+        need = heads * dim * vdim
+    if state.dim() != 2 or state.shape[1] < need:
+        raise ValueError(f"linear_recurrence: a state slot needs {need} elements")
+    if max(q_off, k_off) + heads * dim > proj.shape[1] or v_off + heads * vdim > proj.shape[1] or out.shape[1] != heads * vdim:
+        raise ValueError("linear_recurrence: projections or out do not fit")
+    if seq_rows.numel() < 2 * nseq or slots.numel() < nseq:
+        raise ValueError("linear_recurrence: fewer request records than requests")
+    _check(_fn("bw_linear_recurrence")(int(mode), proj.data_ptr(), proj.stride(0), q_off, k_off, v_off, gate.data_ptr(),
+                                       gate.stride(0), gate_off, gate2_off, bias.data_ptr(),
+                                       0 if bias2 is None else bias2.data_ptr(), float(param), float(qscale), state.data_ptr(),
+                                       state.stride(0), out.data_ptr(), out.stride(0), seq_rows.data_ptr(), slots.data_ptr(),
+                                       positions.data_ptr(), nseq, heads, dim, vdim, _stream()), "linear_recurrence")
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, per_head_weight: bool, g: torch.Tensor, g_off: int, gate: int,
+                   out: torch.Tensor, positions: torch.Tensor, rows: int, heads: int, vdim: int, eps: float) -> None:
+    """out[r, h] = o[r, h] / rms(o[r, h]) * weight * gate(g[r, g_off + h*vdim ..]); weight [heads*vdim] or [vdim]."""
+    _need(o, torch.float32, "o")
+    _need(weight, torch.float32, "weight")
+    _need(g, torch.float32, "g")
+    _need(positions, torch.int32, "positions")
+    if weight.numel() != (heads * vdim if per_head_weight else vdim) or o.shape[1] != heads * vdim or out.shape[1] != heads * vdim:
+        raise ValueError("head_norm_gate: weight, o or out do not fit heads x vdim")
+    if g_off + heads * vdim > g.shape[1] or min(o.shape[0], out.shape[0], g.shape[0], positions.numel()) < rows:
+        raise ValueError("head_norm_gate: buffers too small")
+    gp = g.data_ptr() + 4 * g_off
+    _check(_fn("bw_head_norm_gate")(o.data_ptr(), o.stride(0), weight.data_ptr(), vdim if per_head_weight else 0, gp, g.stride(0),
+                                    int(gate), out.data_ptr(), _act_out(out, "out"), out.stride(0), positions.data_ptr(), rows,
+                                    heads, vdim, float(eps), _stream()), "head_norm_gate")
+
+
+def glu(gate_up: torch.Tensor, out: torch.Tensor, rows: int, act: int) -> None:
+    """out = act(gate) * up of the stacked 32-bit product [rows, 2*inter]; out float32 or bfloat16 (one rounding)."""
+    _need(gate_up, torch.float32, "gate_up")
+    inter = out.shape[1]
+    if gate_up.shape[1] != 2 * inter or gate_up.shape[0] < rows or out.shape[0] < rows:
+        raise ValueError("glu: gate_up must be [rows, 2*inter] for out [rows, inter]")
+    _check(_fn("bw_glu")(gate_up.data_ptr(), out.data_ptr(), _act_out(out, "out"), rows, inter, int(act), _stream()), "glu")
+
+
+# ------------------------------------------------------------------------------ attention over a compressed cache
+
+def latent_prep(proj: torch.Tensor, q_off: int, dkv_off: int, norm_w: torch.Tensor, eps: float, cos: torch.Tensor,
+                sin: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
+                cache: torch.Tensor, qa: torch.Tensor, rows: int, heads: int, dim: int, rot: int, rotary: int, rank: int,
+                page_size: int, write_cache: bool = True) -> None:
+    """From the stacked projections: the latent (RMS-normed) and the rotated shared key part into the row's page slot
+    ([pages, page_size * (rank + rot)]), and every head's rotated query part into ``qa`` [rows, heads * (rank + rot)]
+    behind the place of its latent-space part."""
+    _need(proj, torch.float32, "proj")
+    _need(norm_w, torch.float32, "norm weight")
+    _need(cos, torch.float32, "cos table")
+    _need(sin, torch.float32, "sin table")
+    _need(qa, torch.float32, "qa")
+    for t, what in ((positions, "positions"), (row_seq, "row_seq"), (block_table, "block_table")):
+        _need(t, torch.int32, what)
+    width = rank + rot
+    if q_off + heads * (dim + rot) > proj.shape[1] or dkv_off + width > proj.shape[1] or norm_w.numel() != rank:
+        raise ValueError("latent_prep: projections or norm weight do not fit")
+    if rotary % 2 or rotary > rot or (rotary and (cos.shape[1] != rotary // 2 or sin.shape != cos.shape)):
+        raise ValueError("latent_prep: rotary tables must be [positions, rotary/2]")
+    if cache.dim() != 2 or cache.shape[1] != page_size * width or qa.shape[1] != heads * width:
+        raise ValueError("latent_prep: cache pages or qa do not fit")
+    if min(proj.shape[0], qa.shape[0], positions.numel(), row_seq.numel()) < rows:
+        raise ValueError("latent_prep: buffers shorter than the rows")
+    _check(_fn("bw_latent_prep")(proj.data_ptr(), proj.stride(0), q_off, dkv_off, norm_w.data_ptr(), float(eps), cos.data_ptr(),
+                                 sin.data_ptr(), positions.data_ptr(), row_seq.data_ptr(), block_table.data_ptr(),
+                                 block_table.stride(0), cache.data_ptr(), _act_out(cache, "cache"), qa.data_ptr(), qa.stride(0),
+                                 rows, heads, dim, rot, rotary, rank, page_size, int(write_cache), _stream()), "latent_prep")
+
+
+def headwise_linear(x: torch.Tensor, x_off: int, x_head_stride: int, wt: torch.Tensor, out: torch.Tensor, out_off: int,
+                    out_head_stride: int, rows: int) -> None:
+    """out[r, out_off + h*out_head_stride + o] = sum_i wt[h, i, o] * x[r, x_off + h*x_head_stride + i]: a product per head,
+    weights input-major [heads, in, out] (bfloat16 or float32), 32-bit sums."""
+    _need(x, torch.float32, "x")
+    if wt.dim() != 3 or not wt.is_cuda or not wt.is_contiguous():
+        raise ValueError("headwise_linear: weights must be a contiguous [heads, in, out] GPU tensor")
+    heads, inn, outn = wt.shape
+    if x_off + (heads - 1) * x_head_stride + inn > x.shape[1] or out_off + (heads - 1) * out_head_stride + outn > out.shape[1]:
+        raise ValueError("headwise_linear: x or out narrower than the heads need")
+    if x.shape[0] < rows or out.shape[0] < rows:
+        raise ValueError("headwise_linear: buffers shorter than the rows")
+    ob = _act_out(out, "out")
+    _check(_fn("bw_headwise_linear")(x.data_ptr() + 4 * x_off, x.stride(0), x_head_stride, wt.data_ptr(), _is_bf16(wt, "weights"),
+                                     inn, outn, out.data_ptr() + (2 if ob else 4) * out_off, ob, out.stride(0), out_head_stride,
+                                     rows, heads, _stream()), "headwise_linear")
+
+
+def shared_key_attention(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, tiles: Optional[torch.Tensor],
+                         num_tiles: int, cache: torch.Tensor, sink: Optional[torch.Tensor], out: torch.Tensor, heads: int,
+                         dk: int, dv: int, page_size: int, window: int, scale: float, heads_per_group: int) -> None:
+    """Causal softmax attention of ``heads`` query heads over keys that all heads share: q [rows, heads*dk], cache
+    [pages, page_size*dk] (a token's value is the first dv elements of its key vector), out [rows, heads*dv] (32-bit).
+    ``sink`` [heads]: a score per head that joins the softmax's denominator and has no value.  tiles [n, 4] = (first
+    row, rows, request, 0) with up to 16 / heads_per_group rows each; None: tile t is row t of request t."""
+    _need(q, torch.float32, "q")
+    _need(out, torch.float32, "out")
+    _need(positions, torch.int32, "positions")
+    _need(block_table, torch.int32, "block_table")
+    if tiles is not None:
+        _need(tiles, torch.int32, "tiles")
+        if tiles.numel() < 4 * num_tiles:
+            raise ValueError("shared_key_attention: fewer tiles than said")
+    elif positions.numel() < num_tiles or block_table.shape[0] < num_tiles:
+        raise ValueError("shared_key_attention: fewer rows or block tables than implicit tiles")
+    if sink is not None:
+        _need(sink, torch.float32, "sink")
+        if sink.numel() != heads:
+            raise ValueError("shared_key_attention: a sink per head is needed")
+    if q.shape[1] != heads * dk or out.shape[1] != heads * dv or dv > dk or dv > 512:
+        raise ValueError("shared_key_attention: q or out do not fit (values of up to 512 elements)")
+    if cache.dim() != 2 or cache.shape[1] != page_size * dk:
+        raise ValueError(f"shared_key_attention: cache must be [pages, {page_size * dk}]")
+    _check(_fn("bw_shared_key_attention")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
+                                          block_table.stride(0), 0 if tiles is None else tiles.data_ptr(), num_tiles,
+                                          cache.data_ptr(), _act_out(cache, "cache"), cache.shape[0],
+                                          0 if sink is None else sink.data_ptr(), out.data_ptr(), out.stride(0), heads, dk, dv,
+                                          page_size, int(window), float(scale), int(heads_per_group), _stream()),
+           "shared_key_attention")
 
 
 # ------------------------------------------------------------------------------ sampling

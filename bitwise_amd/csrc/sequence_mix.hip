@@ -1,0 +1,357 @@
+// Kernels of mixers that carry a fixed-size state from token to token instead of a paged cache:
+// token shift (fused with the RMSNorm in front of it), the linear recurrence with a matrix state per
+// head (gated linear attention with a decay per key channel, and the mLSTM with scalar gates, a
+// normaliser and a running maximum), the per-head RMS norm with an output gate behind it, and the
+// gated unit of a feed-forward with a choice of activation.
+//
+// Everything here is 32-bit arithmetic whatever the mode: the state, the gates, their logarithms and
+// exponentials, the norms.  The mode only decides the dtype of what is handed to the next matrix product.
+//
+// A step's rows of one request are consecutive and in position order; ``seq_rows`` holds for every
+// request of the step (first row, number of rows) and ``slots`` its state slot.  A request with no rows,
+// a negative slot or a negative first position is padding and is skipped: its state is not touched.
+#include "common.h"
+#include "api.h"
+
+#include <math.h>
+
+namespace {
+
+__device__ __forceinline__ float log_sigmoid(float z) {
+  // log(1 / (1 + e^-z)) = min(z, 0) - log1p(e^-|z|)
+  return fminf(z, 0.0f) - log1pf(bw_expf(-fabsf(z)));
+}
+
+template <typename OT>
+__device__ __forceinline__ void store_act(OT* p, float v) {
+  if constexpr (sizeof(OT) == 2) *p = f32_to_bf16(v);
+  else *p = v;
+}
+
+// Sum of squares of a row: lane l runs one fused multiply-add chain over elements l, l+64, ... in ascending order,
+// the lanes are joined by the butterflies of wave_sum.  The order depends on the width alone.
+__device__ __forceinline__ float row_sumsq(const float* __restrict__ xr, int dim, int lane) {
+  float acc = 0.0f;
+  for (int i = lane; i < dim; i += 64) acc = fmaf(xr[i], xr[i], acc);
+  return wave_sum(acc);
+}
+
+// ------------------------------------------------------------------------- RMSNorm + token shift
+
+// out[r] = h[r] + (h'[r] - h[r]) * mix with h = (x * inv_rms) * w and h' the h of the request's previous token: the
+// row above, or for the first row of a request in this step what the state slot holds (zeros for a new request).
+// The wave of a request's first row also leaves the h of the request's last row in the slot, after it has read it:
+// nothing else reads or writes that slot in this launch.  A wave a row.
+template <typename OT>
+__global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                         const float* __restrict__ mix, float* __restrict__ state,
+                                                         long long state_ld, const int32_t* __restrict__ positions,
+                                                         const int32_t* __restrict__ row_seq,
+                                                         const int32_t* __restrict__ seq_rows,
+                                                         const int32_t* __restrict__ slots, OT* __restrict__ out, int ldo,
+                                                         int rows, int dim, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * (blockDim.x >> 6) + wave_index();
+  if (row >= rows) return;
+  if (positions[row] < 0) return;
+  const int seq = row_seq[row];
+  const int first = seq_rows[2 * seq], count = seq_rows[2 * seq + 1];
+  const int slot = slots[seq];
+  if (slot < 0 || count <= 0) return;
+  const float* xr = x + (size_t)row * ldx;
+  const float inv = 1.0f / sqrtf(row_sumsq(xr, dim, lane) / (float)dim + eps);
+  float* st = state + (size_t)slot * state_ld;
+  OT* o = out + (size_t)row * ldo;
+  if (row != first) {
+    const float* xp = xr - ldx;
+    const float invp = 1.0f / sqrtf(row_sumsq(xp, dim, lane) / (float)dim + eps);
+    for (int i = lane; i < dim; i += 64) {
+      const float h = (xr[i] * inv) * w[i];
+      const float hp = (xp[i] * invp) * w[i];
+      store_act(o + i, fmaf(hp - h, mix[i], h));
+    }
+    return;
+  }
+  const int last = first + count - 1;
+  const float* xl = x + (size_t)last * ldx;
+  const float invl = last == row ? inv : 1.0f / sqrtf(row_sumsq(xl, dim, lane) / (float)dim + eps);
+  for (int i = lane; i < dim; i += 64) {
+    const float h = (xr[i] * inv) * w[i];
+    const float hp = st[i];
+    store_act(o + i, fmaf(hp - h, mix[i], h));
+    st[i] = (xl[i] * invl) * w[i];
+  }
+}
+
+// ------------------------------------------------------------------------- the linear recurrence
+
+enum { RECUR_DECAY_PER_CHANNEL = 0, RECUR_SCALAR_GATES = 1 };
+
+struct RecurArgs {
+  const float* proj;       // [rows, ldp]: the rows' stacked projections
+  int ldp, q_off, k_off, v_off;
+  const float* gate;       // per channel: decay logits [rows, ldg] at gate_off + head*dim + d;
+  int ldg, gate_off, gate2_off;   // scalar gates: input gate at gate_off + head, forget gate at gate2_off + head
+  const float* bias;       // per channel: [heads*dim]; scalar gates: input-gate bias [heads]
+  const float* bias2;      // scalar gates: forget-gate bias [heads]
+  float param;             // per channel: 1 / tau; scalar gates: the cap
+  float qscale;
+  float* state;            // [slots, state_ld]: S [heads][dim][vdim]; scalar gates also n [heads][dim] and m [heads]
+  long long state_ld;
+  float* out;              // [rows, ldo]: head h at columns h*vdim ..
+  int ldo;
+  const int32_t* seq_rows;
+  const int32_t* slots;
+  const int32_t* positions;
+  int heads, dim, vdim;
+};
+
+// One wave per (request, head, block of 64 value columns).  Lane j keeps column j of the head's state matrix in
+// registers (one element per key channel), so the read-out S^T q needs no exchange between lanes; the tokens' q, k and
+// decays come through LDS in chunks of RC tokens and are read from there by all lanes at once.
+//
+// RECUR_DECAY_PER_CHANNEL:  S[d][j] <- alpha[d] S[d][j] + k[d] v[j],  alpha = exp(logsigmoid(z + bias) / tau);  o[j] = sum_d S[d][j] q[d].
+// RECUR_SCALAR_GATES:  i = cap tanh((gi + bi) / cap), f = logsigmoid(cap tanh((gf + bf) / cap)), m' = max(f + m, i),
+//   S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k alone, o[j] = (S^T q)[j] / (max(|n.q|, e^-m') + 1e-6).
+//   n is spread over the lanes (lane l holds n[l], n[l+64], ...); every wave of a head computes it, the wave of
+//   column block 0 stores it.
+#define RC 16
+template <int MODE, int DPAD>
+__global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
+  constexpr bool GATES = MODE == RECUR_SCALAR_GATES;
+  constexpr int NN = (DPAD + 63) / 64;
+  __shared__ float qs[RC][DPAD];
+  __shared__ float ks[RC][DPAD];
+  __shared__ float as[GATES ? 1 : RC][GATES ? 1 : DPAD];
+  __shared__ float gi[RC], gf[RC];
+  __shared__ float vs[RC][64];
+  const int lane = threadIdx.x;
+  const int cb = blockIdx.x, h = blockIdx.y, s = blockIdx.z;
+  const int first = a.seq_rows[2 * s], count = a.seq_rows[2 * s + 1];
+  const int slot = a.slots[s];
+  if (count <= 0 || slot < 0) return;
+  if (a.positions[first] < 0) return;
+  const int dim = a.dim, vdim = a.vdim;
+  const int j = cb * 64 + lane;
+  const bool live = j < vdim;
+  float* st = a.state + (size_t)slot * a.state_ld;
+  float* S = st + (size_t)h * dim * vdim;
+  float* nv = st + (size_t)a.heads * dim * vdim + (size_t)h * dim;
+  float* mv = st + (size_t)a.heads * dim * vdim + (size_t)a.heads * dim + h;
+
+  float Sreg[DPAD];
+#pragma unroll
+  for (int d = 0; d < DPAD; ++d) Sreg[d] = (live && d < dim) ? S[(size_t)d * vdim + j] : 0.0f;
+  float nreg[NN];
+  float m = 0.0f;
+  if constexpr (GATES) {
+#pragma unroll
+    for (int i = 0; i < NN; ++i) nreg[i] = (lane + 64 * i < dim) ? nv[lane + 64 * i] : 0.0f;
+    m = *mv;
+  }
+
+  for (int t0 = 0; t0 < count; t0 += RC) {
+    const int tc = min(RC, count - t0);
+    __syncthreads();
+    for (int e = lane; e < tc * DPAD; e += 64) {
+      const int t = e / DPAD, d = e % DPAD;
+      const size_t row = (size_t)(first + t0 + t);
+      const float* pr = a.proj + row * a.ldp;
+      const bool in = d < dim;
+      qs[t][d] = in ? pr[a.q_off + h * dim + d] * a.qscale : 0.0f;
+      ks[t][d] = in ? pr[a.k_off + h * dim + d] : 0.0f;
+      if constexpr (!GATES) {
+        float al = 0.0f;
+        if (in) {
+          const float z = a.gate[row * a.ldg + a.gate_off + h * dim + d] + a.bias[h * dim + d];
+          al = bw_expf(log_sigmoid(z) * a.param);
+        }
+        as[t][d] = al;
+      }
+    }
+    if constexpr (GATES) {
+      if (lane < tc) {
+        const float* pr = a.proj + (size_t)(first + t0 + lane) * a.ldp;
+        const float cap = a.param;
+        gi[lane] = cap * tanhf((pr[a.gate_off + h] + a.bias[h]) / cap);
+        gf[lane] = log_sigmoid(cap * tanhf((pr[a.gate2_off + h] + a.bias2[h]) / cap));
+      }
+    }
+    // (each lane writes and reads its own column of vs)
+#pragma unroll
+    for (int t = 0; t < RC; ++t)
+      vs[t][lane] = (live && t < tc) ? a.proj[(size_t)(first + t0 + t) * a.ldp + a.v_off + h * vdim + j] : 0.0f;
+    __syncthreads();
+    for (int t = 0; t < tc; ++t) {
+      float o = 0.0f;
+      if constexpr (!GATES) {
+        const float v = vs[t][lane];
+#pragma unroll
+        for (int d = 0; d < DPAD; ++d) {
+          Sreg[d] = fmaf(as[t][d], Sreg[d], ks[t][d] * v);
+          o = fmaf(Sreg[d], qs[t][d], o);
+        }
+      } else {
+        const float ig = gi[t], fg = gf[t];
+        const float mn = fmaxf(fg + m, ig);
+        const float fa = bw_expf(fg + m - mn);
+        const float ib = bw_expf(ig - mn);
+        m = mn;
+        const float bv = ib * vs[t][lane];
+#pragma unroll
+        for (int d = 0; d < DPAD; ++d) {
+          Sreg[d] = fmaf(fa, Sreg[d], ks[t][d] * bv);
+          o = fmaf(Sreg[d], qs[t][d], o);
+        }
+        float part = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NN; ++i) {
+          const int d = lane + 64 * i;
+          if (d < DPAD) {
+            nreg[i] = fmaf(fa, nreg[i], ib * ks[t][d]);
+            part = fmaf(nreg[i], qs[t][d], part);
+          }
+        }
+        const float nq = wave_sum(part);
+        o = o / (fmaxf(fabsf(nq), bw_expf(-mn)) + 1e-6f);
+      }
+      if (live) a.out[(size_t)(first + t0 + t) * a.ldo + h * vdim + j] = o;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int d = 0; d < DPAD; ++d)
+      if (d < dim) S[(size_t)d * vdim + j] = Sreg[d];
+  }
+  if constexpr (GATES) {
+    if (cb == 0) {
+#pragma unroll
+      for (int i = 0; i < NN; ++i)
+        if (lane + 64 * i < dim) nv[lane + 64 * i] = nreg[i];
+      if (lane == 0) *mv = m;
+    }
+  }
+}
+
+template <int MODE>
+int launch_recurrence(const RecurArgs& a, int nseq, hipStream_t s) {
+  const dim3 grid((a.vdim + 63) / 64, a.heads, nseq), block(64);
+  if (a.dim <= 16) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 16>), grid, block, 0, s, a);
+  else if (a.dim <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 32>), grid, block, 0, s, a);
+  else if (a.dim <= 64) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 64>), grid, block, 0, s, a);
+  else if (a.dim <= 128) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 128>), grid, block, 0, s, a);
+  else return -4;
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------- per-head RMS norm and output gate
+
+enum { GATE_SIGMOID = 0, GATE_SILU = 1 };
+
+// out[r][h*vdim + j] = o[r][h][j] / sqrt(mean_j o^2 + eps) * weight[h*wstride + j] * gate(g[r][h*vdim + j]); a wave per (row, head).
+template <typename OT>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, int ldi, const float* __restrict__ weight,
+                                                             int wstride, const float* __restrict__ g, int ldg, int gate,
+                                                             OT* __restrict__ out, int ldo, const int32_t* __restrict__ positions,
+                                                             int rows, int heads, int vdim, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * (blockDim.x >> 6) + wave_index();
+  if (item >= rows * heads) return;
+  const int row = item / heads, h = item % heads;
+  if (positions[row] < 0) return;
+  const float* orow = o + (size_t)row * ldi + h * vdim;
+  const float inv = 1.0f / sqrtf(row_sumsq(orow, vdim, lane) / (float)vdim + eps);
+  const float* grow = g + (size_t)row * ldg + h * vdim;
+  const float* wr = weight + (size_t)h * wstride;
+  OT* dst = out + (size_t)row * ldo + h * vdim;
+  for (int jj = lane; jj < vdim; jj += 64) {
+    const float z = grow[jj];
+    const float sg = 1.0f / (1.0f + bw_expf(-z));
+    const float gv = gate == GATE_SILU ? z * sg : sg;
+    store_act(dst + jj, ((orow[jj] * inv) * wr[jj]) * gv);
+  }
+}
+
+// ------------------------------------------------------------------------- gated unit
+
+enum { ACT_SILU = 0, ACT_GELU_TANH = 1 };
+
+template <typename OT>
+__global__ void glu_kernel(const float* __restrict__ gu, OT* __restrict__ hout, long long n, int inter, int act) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const long long row = idx / inter;
+  const int c = (int)(idx % inter);
+  const float g = gu[row * 2 * inter + c], u = gu[row * 2 * inter + inter + c];
+  float ag;
+  if (act == ACT_GELU_TANH) {
+    const float inner = 0.7978845608028654f * (g + 0.044715f * ((g * g) * g));
+    ag = (0.5f * g) * (1.0f + tanhf(inner));
+  } else {
+    ag = g * (1.0f / (1.0f + bw_expf(-g)));
+  }
+  store_act(hout + idx, ag * u);
+}
+
+}  // namespace
+
+extern "C" int bw_norm_shift(const float* x, int ldx, const float* w, const float* mix, float* state, long long state_ld,
+                             const int32_t* positions, const int32_t* row_seq, const int32_t* seq_rows,
+                             const int32_t* slots, void* out, int out_is_bf16, int ldo, int rows, int dim, float eps,
+                             void* stream) {
+  if (rows <= 0) return 0;
+  if (dim <= 0 || ldx < dim || ldo < dim || state_ld < dim) return -2;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((rows + 3) / 4), block(256);
+  if (out_is_bf16)
+    hipLaunchKernelGGL(norm_shift_kernel<bf16_t>, grid, block, 0, s, x, ldx, w, mix, state, state_ld, positions, row_seq,
+                       seq_rows, slots, (bf16_t*)out, ldo, rows, dim, eps);
+  else
+    hipLaunchKernelGGL(norm_shift_kernel<float>, grid, block, 0, s, x, ldx, w, mix, state, state_ld, positions, row_seq,
+                       seq_rows, slots, (float*)out, ldo, rows, dim, eps);
+  return BW_LAUNCH_CHECK();
+}
+
+extern "C" int bw_linear_recurrence(int mode, const float* proj, int ldp, int q_off, int k_off, int v_off, const float* gate,
+                                    int ldg, int gate_off, int gate2_off, const float* bias, const float* bias2, float param,
+                                    float qscale, float* state, long long state_ld, float* out, int ldo,
+                                    const int32_t* seq_rows, const int32_t* slots, const int32_t* positions, int nseq,
+                                    int heads, int dim, int vdim, void* stream) {
+  if (nseq <= 0) return 0;
+  if (heads <= 0 || dim <= 0 || vdim <= 0 || ldo < heads * vdim) return -2;
+  const long long need = (long long)heads * dim * vdim + (mode == RECUR_SCALAR_GATES ? (long long)heads * dim + heads : 0);
+  if (state_ld < need) return -2;
+  RecurArgs a{proj, ldp, q_off, k_off, v_off, gate, ldg, gate_off, gate2_off, bias, bias2, param, qscale, state, state_ld,
+              out, ldo, seq_rows, slots, positions, heads, dim, vdim};
+  hipStream_t s = (hipStream_t)stream;
+  if (mode == RECUR_SCALAR_GATES) return launch_recurrence<RECUR_SCALAR_GATES>(a, nseq, s);
+  if (mode == RECUR_DECAY_PER_CHANNEL) return launch_recurrence<RECUR_DECAY_PER_CHANNEL>(a, nseq, s);
+  return -2;
+}
+
+extern "C" int bw_head_norm_gate(const float* o, int ldi, const float* weight, int wstride, const float* g, int ldg, int gate,
+                                 void* out, int out_is_bf16, int ldo, const int32_t* positions, int rows, int heads, int vdim,
+                                 float eps, void* stream) {
+  if (rows <= 0) return 0;
+  if (heads <= 0 || vdim <= 0 || ldi < heads * vdim || ldo < heads * vdim) return -2;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((rows * heads + 3) / 4), block(256);
+  if (out_is_bf16)
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, s, o, ldi, weight, wstride, g, ldg, gate, (bf16_t*)out,
+                       ldo, positions, rows, heads, vdim, eps);
+  else
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, s, o, ldi, weight, wstride, g, ldg, gate, (float*)out,
+                       ldo, positions, rows, heads, vdim, eps);
+  return BW_LAUNCH_CHECK();
+}
+
+extern "C" int bw_glu(const float* gate_up, void* h, int out_is_bf16, int rows, int inter, int act, void* stream) {
+  if (rows <= 0 || inter <= 0) return 0;
+  if (act != ACT_SILU && act != ACT_GELU_TANH) return -2;
+  const long long n = (long long)rows * inter;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  if (out_is_bf16) hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, block, 0, s, gate_up, (bf16_t*)h, n, inter, act);
+  else hipLaunchKernelGGL(glu_kernel<float>, grid, block, 0, s, gate_up, (float*)h, n, inter, act);
+  return BW_LAUNCH_CHECK();
+}

@@ -80,12 +80,13 @@ class StepContext:
                 t[i, :len(row)] = np.maximum(row, 0)      # pages given back (-1) are never read
             tables.append(t)
         slots = np.asarray([s.slot for s in self.segments], np.int32)
-        parts = [tokens, positions, row_seq, np.asarray(want, np.int32), slots] + [t.reshape(-1) for t in tables]
+        seq_rows = np.asarray([(self.seq_start[i], len(s.tokens)) for i, s in enumerate(self.segments)], np.int32).reshape(-1)
+        parts = [tokens, positions, row_seq, np.asarray(want, np.int32), slots, seq_rows] + [t.reshape(-1) for t in tables]
         packed = torch.from_numpy(np.concatenate(parts)).to(device)
         cuts = np.cumsum([0] + [p.size for p in parts])
         view = [packed[cuts[i]:cuts[i + 1]] for i in range(len(parts))]
-        self.tokens, self.positions, self.row_seq, self.want_rows, self.slots = view[:5]
-        self.block_tables = [view[5 + g].view(nseq, widths[g]) for g in range(num_groups)]
+        self.tokens, self.positions, self.row_seq, self.want_rows, self.slots, self.seq_rows = view[:6]    # seq_rows: (first row, rows) per request
+        self.block_tables = [view[6 + g].view(nseq, widths[g]) for g in range(num_groups)]
         self.host_positions = positions
         self._memo: Dict[Any, Any] = {}
 

@@ -131,7 +131,7 @@ class GpuExecutor:
         self._prints_dev = [torch.zeros(max_logit_rows, dtype=torch.int64, device=rt.device) for _ in range(2)]
         self._prints_in = torch.zeros(max_logit_rows, dtype=torch.int64, device=rt.device)
         self.group_specs = [GroupSpec(g.window) for g in asm.group_specs]
-        self.has_state = bool(asm.state_specs)
+        self.has_state = asm.has_state
         self.prefix_reusable = asm.prefix_reusable      # every mixer keeps what it computed in its pages
         self.run_ahead_safe = asm.run_ahead_safe        # no mixer minds a row that runs for a request that has ended
         self.vocab_size = asm.spec.vocab_size

@@ -65,6 +65,7 @@ class _StaticDecodeContext:
         # row: the next step of the same requests in the same order can be launched before the host has the tokens
         self.token_feedback = self.sampled
         self.row_seq = torch.arange(size, dtype=torch.int32, device=device)
+        self.seq_rows = torch.stack([self.row_seq, torch.ones_like(self.row_seq)], dim=1).contiguous().view(-1)   # (row t, 1 row)
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
         self.segments: List[Segment] = []
         self.seq_start = list(range(size))

@@ -33,16 +33,19 @@ class CacheStorage:
         self.states: Dict[int, torch.Tensor] = {}
         for idx, ss in model.state_specs.items():
             self.states[idx] = torch.zeros((self.num_slots, *ss.shape), dtype=_TORCH_DTYPE[ss.dtype], device=rt.device)
+        self.block_states: Dict[int, torch.Tensor] = {}
+        for idx, ss in model.block_state_specs.items():
+            self.block_states[idx] = torch.zeros((self.num_slots, *ss.shape), dtype=_TORCH_DTYPE[ss.dtype], device=rt.device)
         self.bindings: List[CallBinding] = []
         for plan in model.calls:
-            call = dataclasses.replace(plan, state=self.states.get(plan.index))
+            call = dataclasses.replace(plan, state=self.states.get(plan.index), block_state=self.block_states.get(plan.index))
             if call.group >= 0:
                 call.k_cache = self.keys[call.group][call.cache_index]
                 call.v_cache = self.values[call.group][call.cache_index]
             self.bindings.append(call)
 
     def nbytes(self) -> int:
-        tensors = self.keys + self.values + list(self.states.values())
+        tensors = self.keys + self.values + list(self.states.values()) + list(self.block_states.values())
         return sum(t.numel() * t.element_size() for t in tensors)
 
     def bytes_per_token(self) -> int:
@@ -54,7 +57,7 @@ class CacheStorage:
 
     def reset_slot(self, slot: int) -> None:
         """Fixed-size state starts from zero when a request takes the slot."""
-        for t in self.states.values():
+        for t in list(self.states.values()) + list(self.block_states.values()):
             t[slot].zero_()
 
     def poison_pages(self, group: int, pages) -> None:

@@ -54,7 +54,7 @@ class Model:
     def load(cls, path: str | Path, dtype: str = "bfloat16", device: str = "cuda:0") -> "Model":
         """``path``: a folder with config.json and *.safetensors; the model class is chosen by
         ``architectures[0]``.  dtype "bfloat16" or "float32" picks the precision mode."""
-        raw = registry.read_config(path)
+        raw = registry.read_model_config(path)
         arch = registry.architecture_of(raw)
         typed = arch.config_from_dict(raw)
         rt = Runtime(dtype, device)
@@ -89,7 +89,7 @@ class Model:
                 tensors[name] = torch.randint(0, 2 ** 15, ts.shape, generator=gen, dtype=torch.int32, device=rt.device)
                 continue
             z = torch.randn(ts.shape, generator=gen, dtype=torch.float32, device=rt.device)
-            tensors[name] = ((1.0 + 0.1 * z) if ts.kind == "norm" else (sigma * z)).to(wd)
+            tensors[name] = loader.shape_values(ts.kind, z, sigma).to(wd)
         assembled.bind_tensors(tensors)
         return cls(typed, assembled)
 

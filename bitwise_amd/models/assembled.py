@@ -29,6 +29,7 @@ class CallBinding:
     k_cache: Optional[torch.Tensor] = None
     v_cache: Optional[torch.Tensor] = None
     state: Optional[torch.Tensor] = None
+    block_state: Optional[torch.Tensor] = None     # state of the layer's arrangement itself (parts.base.Block.state_spec)
 
 
 class AssembledModel:
@@ -56,8 +57,14 @@ class AssembledModel:
         self.launches_through_ops = all(getattr(p, "launches_through_ops", False) for p in every)
         # each mixer's own word on what the engine may do around it (parts.base.Mixer)
         mixers = [self.layers[c.layer].mixer for c in spec.schedule]
-        self.prefix_reusable = all(m.prefix_reusable for m in mixers)
-        self.run_ahead_safe = all(m.run_ahead_safe for m in mixers)
+        stateless_blocks = not self.block_state_specs
+        self.prefix_reusable = stateless_blocks and all(m.prefix_reusable for m in mixers)
+        self.run_ahead_safe = stateless_blocks and all(m.run_ahead_safe for m in mixers)
+
+    @property
+    def has_state(self) -> bool:
+        """Whether a request holds anything outside its pages (a slot of some mixer's or arrangement's state)."""
+        return bool(self.state_specs or self.block_state_specs)
 
     def check_page_size(self, page_size: int) -> None:
         """Refuse a page size that one of the mixers' kernels does not take."""
@@ -73,7 +80,8 @@ class AssembledModel:
         self.group_caches: List[List[int]] = []          # group -> cache numbers, in storage order
         cache_home: Dict[int, Tuple[int, int]] = {}       # cache number -> (group, index in group)
         self.calls: List[CallBinding] = []
-        self.state_specs: Dict[int, StateSpec] = {}       # call index -> per-request state
+        self.state_specs: Dict[int, StateSpec] = {}       # call index -> per-request state of the mixer
+        self.block_state_specs: Dict[int, StateSpec] = {} # call index -> per-request state of the arrangement
         for idx, c in enumerate(schedule):
             if not 0 <= c.layer < len(self.layers):
                 raise ValueError(f"schedule entry {idx} names layer {c.layer}, the model has {len(self.layers)}")
@@ -100,6 +108,9 @@ class AssembledModel:
             ss = mixer.state_spec()
             if ss is not None:
                 self.state_specs[idx] = ss
+            bs = self.layers[c.layer].state_spec()
+            if bs is not None:
+                self.block_state_specs[idx] = bs
             self.calls.append(CallBinding(idx, c.layer, c.cache, group, cindex, c.writes_cache))
 
     # ------------------------------------------------------------------ tensors

@@ -20,8 +20,9 @@ from typing import Any, Callable, Dict, List, Optional, Tuple, Type
 class TensorSpec:
     """One checkpoint tensor a part needs: its shape and what kind of values it holds.
 
-    kind: "linear" / "embedding" (random init N(0, sigma)), "norm" (1 + N(0, 0.1)) or
-    "int" (integer table, kept as int32).
+    kind: "linear" / "embedding" (random init N(0, sigma)), "norm" (1 + N(0, 0.1)),
+    "around_zero" (N(0, 0.1): a norm weight stored as its distance from 1), "unit_interval" (a mixing
+    weight in (0, 1)), "bias" (N(0, 1): gate biases, sinks) or "int" (integer table, kept as int32).
     """
     shape: Tuple[int, ...]
     kind: str = "linear"
@@ -161,6 +162,11 @@ class Head(Part):
 
 
 class Norm(Part):
+    def state_spec(self) -> Optional["StateSpec"]:
+        """Per-request state of a norm that mixes a request's previous token into its output; None: it has none.  The
+        block that owns the norm asks for it and hands the bound tensor back with every call (``state``)."""
+        return None
+
     def forward(self, ctx, x):
         """x: [rows, width] 32-bit residual stream -> normed rows in the activation dtype."""
         raise NotImplementedError
@@ -247,16 +253,21 @@ class Block(Part):
     names.  Every arrangement has a role "mixer"."""
 
     roles: Dict[str, str] = {}
+    optional_roles: Tuple[str, ...] = ()      # roles a layer may leave out (the attribute is None then)
 
     def __init__(self, parts: Dict[str, Part], runtime):
         super().__init__({}, runtime)
-        missing = [r for r in self.roles if r not in parts]
+        missing = [r for r in self.roles if r not in parts and r not in self.optional_roles]
         extra = [r for r in parts if r not in self.roles]
         if missing or extra:
             raise ValueError(f"block {type(self).__name__}: missing parts {missing}, unknown parts {extra}")
-        self.parts = {role: parts[role] for role in self.roles}
-        for role, part in self.parts.items():
-            setattr(self, role, part)
+        self.parts = {role: parts[role] for role in self.roles if role in parts}
+        for role in self.roles:
+            setattr(self, role, self.parts.get(role))
+
+    def state_spec(self) -> Optional[StateSpec]:
+        """Per-request state of the arrangement itself (beside its mixer's): it arrives as ``call.block_state``."""
+        return None
 
     def forward(self, ctx, call, x) -> None:
         raise NotImplementedError

@@ -20,3 +20,35 @@ class PreNormBlock(Block):
         if not self.feed_forward.forward_with_norm(ctx, x, self.ffn_norm, x):
             h = self.ffn_norm.forward(ctx, x)
             self.feed_forward.forward(ctx, h, x)
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """x += mixer(norm1(x)) + feed_forward(norm2(x)), both read the same x; a layer may leave the feed-forward (and its
+    norm) out.  A mixer norm with state of its own (a token shift) gets the call's ``block_state``."""
+
+    roles = {"mixer_norm": "norm", "ffn_norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+    optional_roles = ("ffn_norm", "feed_forward")
+    graph_safe = True
+    launches_through_ops = True
+
+    def __init__(self, parts, runtime):
+        super().__init__(parts, runtime)
+        if (self.feed_forward is None) != (self.ffn_norm is None):
+            raise ValueError("parallel block: a feed-forward and its norm come together or not at all")
+
+    def state_spec(self):
+        return self.mixer_norm.state_spec()
+
+    def forward(self, ctx, call, x) -> None:
+        # both branches' inputs are formed before either adds into x
+        if call.block_state is not None:
+            h = self.mixer_norm.forward(ctx, x, state=call.block_state)
+        else:
+            h = self.mixer_norm.forward(ctx, x, out_name="normed_mixer")
+        if self.feed_forward is not None:
+            # (the fused norm + product reads x before anything is added; the down projection adds afterwards)
+            if not self.feed_forward.forward_with_norm(ctx, x, self.ffn_norm, x):
+                h2 = self.ffn_norm.forward(ctx, x)
+                self.feed_forward.forward(ctx, h2, x)
+        self.mixer.forward(ctx, call, h, x)

@@ -21,13 +21,14 @@ class TokenEmbedding(Embedding):
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
         self.vocab, self.width = int(params["vocab"]), int(params["width"])
+        self.tensor = str(params.get("tensor", "weight"))      # the table's name behind the prefix
         self.weight: Optional[torch.Tensor] = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
-        return {"weight": TensorSpec((self.vocab, self.width), "embedding")}
+        return {self.tensor: TensorSpec((self.vocab, self.width), "embedding")}
 
     def bind(self, tensors) -> None:
-        self.weight = tensors["weight"].to(self.rt.device).contiguous()
+        self.weight = tensors[self.tensor].to(self.rt.device).contiguous()
 
     def weight_bytes(self) -> int:
         return 0      # a step reads one row per token, not the table
@@ -50,10 +51,11 @@ class LMHead(Head):
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
         self.vocab, self.width, self.tied = int(params["vocab"]), int(params["width"]), bool(params["tied"])
+        self.tensor = str(params.get("tensor", "weight"))
         self.linear: Optional[Linear] = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
-        return {} if self.tied else {"weight": TensorSpec((self.vocab, self.width), "linear")}
+        return {} if self.tied else {self.tensor: TensorSpec((self.vocab, self.width), "linear")}
 
     def bind(self, tensors, embedding=None) -> None:
         if self.tied:
@@ -62,7 +64,7 @@ class LMHead(Head):
                 raise ValueError("a tied head needs an embedding part with a table [vocab, width]")
             self.linear = Linear(table, self.rt)     # the same device tensor, not a copy
         else:
-            self.linear = Linear(tensors["weight"], self.rt)
+            self.linear = Linear(tensors[self.tensor], self.rt)
 
     def weight_bytes(self) -> int:
         return self.linear.nbytes()

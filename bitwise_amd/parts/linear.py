@@ -18,7 +18,9 @@ from ..csrc import ops
 
 
 class Linear:
-    def __init__(self, weight: torch.Tensor, runtime, bias: torch.Tensor | None = None):
+    def __init__(self, weight: torch.Tensor, runtime, bias: torch.Tensor | None = None, matrix_cores: bool = True):
+        """``matrix_cores`` False keeps a bfloat16 weight on the 32-bit kernels in bfloat16 mode too (a product whose inner
+        size is tiny, or whose input must not be rounded to bfloat16)."""
         if weight.dim() != 2 or weight.dtype not in (torch.bfloat16, torch.float32):
             raise ValueError("a linear weight must be a bfloat16 or float32 matrix")
         self.rt = runtime
@@ -29,7 +31,7 @@ class Linear:
                 raise ValueError(f"a bias of {tuple(bias.shape)} does not fit a weight of {tuple(weight.shape)}")
             self.bias = bias.to(runtime.device).float().contiguous()      # (widening is exact)
         self.out_features, self.in_features = self.weight.shape
-        self.mfma = runtime.bf16 and self.weight.dtype == torch.bfloat16
+        self.mfma = bool(matrix_cores) and runtime.bf16 and self.weight.dtype == torch.bfloat16
         if self.mfma and self.in_features % 8:
             raise ValueError(f"bfloat16 matrix product: inner size {self.in_features} must be a multiple of 8")
 

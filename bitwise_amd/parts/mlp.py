@@ -1,6 +1,7 @@
-"""Dense SwiGLU feed-forward (src/model.cpp:301-305, src/kernels.cpp:291-298):
-one stacked product [gate; up], h = g * (1/(1+exp(-g))) * u, down projection added into the
-residual stream."""
+"""Dense gated feed-forward (src/model.cpp:301-305, src/kernels.cpp:291-298):
+one stacked product [gate; up], h = act(g) * u, down projection added into the residual stream.
+SwiGLU: act(g) = g * (1/(1+exp(-g))); the gated GELU uses the tanh form
+0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))."""
 
 from __future__ import annotations
 
@@ -15,30 +16,35 @@ from .linear import Linear
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
-    """params: width, inter.  tensors: gate_proj/up_proj/down_proj .weight."""
+    """params: width, inter.  tensors: gate_proj/up_proj/down_proj .weight (or the three names in ``names``)."""
 
     graph_safe = True
     launches_through_ops = True
+    act = ops.ACT_SILU
+    default_names = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
         self.width, self.inter = int(params["width"]), int(params["inter"])
+        self.names = tuple(params.get("names", self.default_names))
+        if len(self.names) != 3:
+            raise ValueError("a gated feed-forward has three tensors: gate, up, down")
         self.gate_up: Optional[Linear] = None
         self.down: Optional[Linear] = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
         return {
-            "gate_proj.weight": TensorSpec((self.inter, self.width)),
-            "up_proj.weight": TensorSpec((self.inter, self.width)),
-            "down_proj.weight": TensorSpec((self.width, self.inter)),
+            self.names[0]: TensorSpec((self.inter, self.width)),
+            self.names[1]: TensorSpec((self.inter, self.width)),
+            self.names[2]: TensorSpec((self.width, self.inter)),
         }
 
     def bind(self, tensors) -> None:
-        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        g, u = tensors[self.names[0]], tensors[self.names[1]]
         if g.dtype != u.dtype:
             raise ValueError("gate and up projections must be stored in one dtype to be stacked")
         self.gate_up = Linear(torch.cat([g, u], dim=0), self.rt)
-        self.down = Linear(tensors["down_proj.weight"], self.rt)
+        self.down = Linear(tensors[self.names[2]], self.rt)
 
     def weight_bytes(self) -> int:
         return self.gate_up.nbytes() + self.down.nbytes()
@@ -72,4 +78,24 @@ class SwiGLU(FeedForward):
                 ops.convert(act32, act, rows)
             else:
                 act = act32
+        self.down.add_into(ws, act, residual, rows)
+
+
+@register_feed_forward("geglu")
+class GeGLU(SwiGLU):
+    """The same arrangement with the tanh form of GELU on the gate.  The stacked product leaves 32-bit sums; the
+    activation and the product with ``up`` are one 32-bit kernel behind it, which rounds once for the down projection."""
+
+    act = ops.ACT_GELU_TANH
+    default_names = ("gate", "up", "down")
+
+    def forward_with_norm(self, ctx, x, norm, residual) -> bool:
+        return False
+
+    def forward(self, ctx, h, residual) -> None:
+        ws, rows = ctx.ws, ctx.rows
+        gu = ws.buffer("gate_up", 2 * self.inter, torch.float32)
+        self.gate_up.store(ws, h, gu, rows)
+        act = ws.buffer("mlp_h", self.inter, self.rt.act_dtype)
+        ops.glu(gu, act, rows, self.act)
         self.down.add_into(ws, act, residual, rows)

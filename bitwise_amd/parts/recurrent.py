@@ -1,0 +1,189 @@
+"""Mixers with a matrix memory per head instead of a cache: S <- decay * S + k v^T, o = S^T q.
+
+Two kinds share the arrangement (one stacked projection of the mixer's input, the recurrence over each request's
+rows in order from and to its state slot, a per-head RMS norm of the read-out with an output gate, the output
+projection added into the residual stream) and differ in the decay:
+
+* ``gla``: gated linear attention, a decay per key channel, alpha = sigmoid(z)^(1/tau) with z a low-rank
+  projection of the input plus a bias; the read-out norm has one weight vector for all heads and the gate is SiLU.
+* ``mlstm``: the matrix memory of the xLSTM, scalar input and forget gates per head in the log domain, capped by
+  cap * tanh(. / cap), with a normaliser n and a running maximum m that starts at 0; the read-out is divided by
+  max(|n.q|, exp(-m)) + 1e-6, the norm weight spans all heads and the gate is a sigmoid.
+
+The state, the gates and everything between the projections and the read-out are 32-bit in both modes; the
+projections' sums arrive as 32-bit values and are not rounded on the way.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..csrc import ops
+from .base import Mixer, StateSpec, TensorSpec, register_mixer
+from .linear import Linear
+
+
+class _MatrixMemoryMixer(Mixer):
+    """params: width, heads, dim (key channels a head), vdim (value channels a head), eps (of the read-out norm);
+    optional ``names``: the tensors' names behind the prefix."""
+
+    graph_safe = True
+    launches_through_ops = True
+    mode = -1
+    gate_kind = ops.GATE_SIGMOID
+    per_head_norm_weight = True
+    stacked: Tuple[str, ...] = ()                # the projections of the input that are stacked into one product
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        p = params
+        self.width, self.heads, self.dim, self.vdim = int(p["width"]), int(p["heads"]), int(p["dim"]), int(p["vdim"])
+        self.eps = float(p["eps"])
+        if self.dim > ops.RECUR_MAX_DIM:
+            raise ValueError(f"{type(self).__name__}: {self.dim} key channels a head; the kernel keeps up to {ops.RECUR_MAX_DIM}")
+        self.qscale = float(self.dim) ** -0.5
+        self.proj: Optional[Linear] = None
+        self.o: Optional[Linear] = None
+        self.norm_weight: Optional[torch.Tensor] = None
+        self.offsets: Dict[str, int] = {}
+        self.proj_width = 0
+
+    # -- sizes of the stacked projections, in order
+    def _stack_sizes(self) -> List[Tuple[str, int]]:
+        raise NotImplementedError
+
+    def _norm_weight_size(self) -> int:
+        return self.heads * self.vdim if self.per_head_norm_weight else self.vdim
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        out = {name: TensorSpec((n, self.width)) for name, n in self._stack_sizes()}
+        out["o"] = TensorSpec((self.width, self.heads * self.vdim))
+        out["norm"] = TensorSpec((self._norm_weight_size(),), "norm")
+        return out
+
+    def _bind_common(self, tensors) -> None:
+        parts = [tensors[name] for name, _ in self._stack_sizes()]
+        if len({t.dtype for t in parts}) != 1:
+            raise ValueError("the projections of one mixer must be stored in one dtype to be stacked")
+        off = 0
+        for name, n in self._stack_sizes():
+            self.offsets[name] = off
+            off += n
+        self.proj_width = off
+        self.proj = Linear(torch.cat(parts, dim=0), self.rt, matrix_cores=self.width % 8 == 0)
+        self.o = Linear(tensors["o"], self.rt, matrix_cores=(self.heads * self.vdim) % 8 == 0)
+        self.norm_weight = tensors["norm"].to(self.rt.device).float().contiguous()
+
+    def state_spec(self) -> StateSpec:
+        n = self.heads * self.dim * self.vdim
+        if self.mode == ops.RECUR_SCALAR_GATES:
+            n += self.heads * self.dim + self.heads
+        return StateSpec((n,), "float32")
+
+    def _project(self, ctx, h) -> torch.Tensor:
+        """The stacked projection of the rows as 32-bit sums."""
+        y = ctx.ws.buffer("recur_proj", self.proj_width, torch.float32)
+        self.proj.store(ctx.ws, h, y, ctx.rows)
+        return y
+
+    def _finish(self, ctx, y, raw, residual) -> None:
+        act = ctx.ws.buffer("recur_gated", self.heads * self.vdim, self.rt.act_dtype)
+        ops.head_norm_gate(raw, self.norm_weight, self.per_head_norm_weight, y, self.offsets["g"], self.gate_kind, act,
+                           ctx.positions, ctx.rows, self.heads, self.vdim, self.eps)
+        self.o.add_into(ctx.ws, act, residual, ctx.rows)
+
+
+@register_mixer("gla")
+class GatedLinearAttention(_MatrixMemoryMixer):
+    """params as the base, plus tau and rank (the inner size of the decay's low-rank projection).
+    tensors: q, k [heads*dim, width]; v, g [heads*vdim, width]; a1 [rank, width]; a2 [heads*dim, rank]; a2.b [heads*dim];
+    norm [vdim]; o [width, heads*vdim]."""
+
+    mode = ops.RECUR_DECAY_PER_CHANNEL
+    gate_kind = ops.GATE_SILU
+    per_head_norm_weight = False
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.tau, self.rank = float(params["tau"]), int(params["rank"])
+        if self.tau <= 0:
+            raise ValueError("gla: tau must be positive")
+        self.a2: Optional[Linear] = None
+        self.a2_bias: Optional[torch.Tensor] = None
+
+    def _stack_sizes(self):
+        hd, hv = self.heads * self.dim, self.heads * self.vdim
+        return [("q", hd), ("k", hd), ("v", hv), ("g", hv), ("a1", self.rank)]
+
+    def tensors(self):
+        out = super().tensors()
+        out["a2"] = TensorSpec((self.heads * self.dim, self.rank))
+        out["a2.b"] = TensorSpec((self.heads * self.dim,), "bias")
+        return out
+
+    def bind(self, tensors) -> None:
+        self._bind_common(tensors)
+        # the inner size is tiny and its input stays 32-bit: the 32-bit kernels in either mode
+        self.a2 = Linear(tensors["a2"], self.rt, matrix_cores=False)
+        self.a2_bias = tensors["a2.b"].to(self.rt.device).float().contiguous()
+
+    def weight_bytes(self) -> int:
+        return self.proj.nbytes() + self.o.nbytes() + self.a2.nbytes() + 4 * (self.a2_bias.numel() + self.norm_weight.numel())
+
+    def forward(self, ctx, call, h, residual) -> None:
+        ws, rows = ctx.ws, ctx.rows
+        y = self._project(ctx, h)
+        low = y[:, self.offsets["a1"]:self.offsets["a1"] + self.rank]      # (a view: the product reads it in place)
+        z = ws.buffer("gla_decay_logits", self.heads * self.dim, torch.float32)
+        self.a2.store(ws, low, z, rows)
+        raw = ws.buffer("recur_out", self.heads * self.vdim, torch.float32)
+        ops.linear_recurrence(self.mode, y, self.offsets["q"], self.offsets["k"], self.offsets["v"], z, 0, 0, self.a2_bias,
+                              None, 1.0 / self.tau, self.qscale, call.state, raw, ctx.seq_rows, ctx.slots, ctx.positions,
+                              ctx.nseq, self.heads, self.dim, self.vdim)
+        self._finish(ctx, y, raw, residual)
+
+
+@register_mixer("mlstm")
+class MatrixLSTM(_MatrixMemoryMixer):
+    """params as the base, plus gate_cap.  tensors: q, k [heads*dim, width]; v, g [heads*vdim, width]; i, f [heads, width];
+    i.b, f.b [heads]; norm [heads*vdim]; o [width, heads*vdim]."""
+
+    mode = ops.RECUR_SCALAR_GATES
+    gate_kind = ops.GATE_SIGMOID
+    per_head_norm_weight = True
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.cap = float(params["gate_cap"])
+        if self.cap <= 0:
+            raise ValueError("mlstm: gate_cap must be positive")
+        self.i_bias: Optional[torch.Tensor] = None
+        self.f_bias: Optional[torch.Tensor] = None
+
+    def _stack_sizes(self):
+        hd, hv = self.heads * self.dim, self.heads * self.vdim
+        return [("q", hd), ("k", hd), ("v", hv), ("g", hv), ("i", self.heads), ("f", self.heads)]
+
+    def tensors(self):
+        out = super().tensors()
+        out["i.b"] = TensorSpec((self.heads,), "bias")
+        out["f.b"] = TensorSpec((self.heads,), "bias")
+        return out
+
+    def bind(self, tensors) -> None:
+        self._bind_common(tensors)
+        self.i_bias = tensors["i.b"].to(self.rt.device).float().contiguous()
+        self.f_bias = tensors["f.b"].to(self.rt.device).float().contiguous()
+
+    def weight_bytes(self) -> int:
+        return self.proj.nbytes() + self.o.nbytes() + 4 * (2 * self.heads + self.norm_weight.numel())
+
+    def forward(self, ctx, call, h, residual) -> None:
+        y = self._project(ctx, h)
+        raw = ctx.ws.buffer("recur_out", self.heads * self.vdim, torch.float32)
+        ops.linear_recurrence(self.mode, y, self.offsets["q"], self.offsets["k"], self.offsets["v"], y, self.offsets["i"],
+                              self.offsets["f"], self.i_bias, self.f_bias, self.cap, self.qscale, call.state, raw,
+                              ctx.seq_rows, ctx.slots, ctx.positions, ctx.nseq, self.heads, self.dim, self.vdim)
+        self._finish(ctx, y, raw, residual)

@@ -9,7 +9,9 @@ from dataclasses import dataclass
 from pathlib import Path
 from typing import Any, Callable, Dict, Mapping, Optional
 
+from .config import kuponex as kuponex_config
 from .config.llama import ConfigError, LlamaConfig
+from .models.kuponex import TINY_KUPONEX, kuponex_spec
 from .models.llama import TINY_LLAMA, llama_spec
 from .parts.base import ModelSpec
 
@@ -20,25 +22,47 @@ class Architecture:
     config_from_dict: Callable[[Mapping[str, Any]], Any]
     spec_from_config: Callable[[Any], ModelSpec]
     tiny_config: Optional[Mapping[str, Any]] = None     # a small config.json of this architecture for simulations and smoke runs
+    # (config, {tensor name: shape}) -> config with the sizes filled in that only the checkpoint's tensor shapes give
+    sizes_from_tensors: Optional[Callable[[Mapping[str, Any], Mapping[str, tuple]], Dict[str, Any]]] = None
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, config_from_dict, spec_from_config, tiny_config=None) -> None:
+def register_architecture(name: str, config_from_dict, spec_from_config, tiny_config=None, sizes_from_tensors=None) -> None:
     if name in ARCHITECTURES:
         raise ValueError(f"architecture '{name}' is already registered")
-    ARCHITECTURES[name] = Architecture(name, config_from_dict, spec_from_config, tiny_config)
+    ARCHITECTURES[name] = Architecture(name, config_from_dict, spec_from_config, tiny_config, sizes_from_tensors)
 
 
 def architecture_of(config: Mapping[str, Any]) -> Architecture:
+    """By ``architectures[0]`` (the exporters' list) or, where a config.json names just one, ``architecture``."""
     archs = config.get("architectures")
-    if not isinstance(archs, (list, tuple)) or not archs:
+    if isinstance(archs, (list, tuple)) and archs:
+        name = archs[0]
+    elif isinstance(config.get("architecture"), str):
+        name = config["architecture"]
+    else:
         raise ConfigError("config.json lacks 'architectures': [name]")
-    arch = ARCHITECTURES.get(archs[0])
+    arch = ARCHITECTURES.get(name)
     if arch is None:
-        raise ConfigError(f"unsupported architecture {archs[0]}; registered: {sorted(ARCHITECTURES)}")
+        raise ConfigError(f"unsupported architecture {name}; registered: {sorted(ARCHITECTURES)}")
     return arch
+
+
+def read_model_config(folder: str | Path) -> Dict[str, Any]:
+    """config.json of a model folder, completed from the shapes in its safetensors headers where the architecture
+    takes sizes from there."""
+    from .weights import safetensors_io
+    raw = read_config(folder)
+    arch = architecture_of(raw)
+    if arch.sizes_from_tensors is not None:
+        shapes: Dict[str, tuple] = {}
+        for shard in sorted(Path(folder).glob("*.safetensors")):
+            header, _ = safetensors_io.read_header(shard)
+            shapes.update({name: tuple(int(s) for s in info["shape"]) for name, info in header.items()})
+        raw = arch.sizes_from_tensors(raw, shapes)
+    return raw
 
 
 def read_config(folder: str | Path) -> Dict[str, Any]:
@@ -49,3 +73,5 @@ def read_config(folder: str | Path) -> Dict[str, Any]:
 
 
 register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec, TINY_LLAMA)
+register_architecture(kuponex_config.ARCHITECTURE, kuponex_config.KuponexConfig.from_dict, kuponex_spec, TINY_KUPONEX,
+                      kuponex_config.sizes_from_tensors)

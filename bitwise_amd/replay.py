@@ -29,7 +29,7 @@ class Replayer:
         rows = max(64, min(int(max_tokens), MAX_STEP_ROWS))
         pages = (int(max_tokens) + block_size - 1) // block_size
         self.manager = CacheManager([GroupSpec(g.window) for g in asm.group_specs], pages, block_size, max_live,
-                                    prefix_caching=False, has_state=bool(asm.state_specs))
+                                    prefix_caching=False, has_state=asm.has_state)
         self.storage = CacheStorage(asm, pages, max_live, block_size)
         max_len = min(asm.spec.max_positions, max(int(max_tokens), 1))
         self.runner = ModelRunner(asm, self.storage, max_model_len=max_len, max_rows=rows, max_logit_rows=rows,

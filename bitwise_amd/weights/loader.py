@@ -83,6 +83,19 @@ def load_folder(folder: str | Path, specs: Mapping[str, TensorSpec], ignored_suf
     return check_and_convert(specs, found, str(folder), ignored_suffixes, unused)
 
 
+def shape_values(kind: str, z: torch.Tensor, sigma: float) -> torch.Tensor:
+    """Standard normals ``z`` turned into the values of a tensor of this kind (parts.base.TensorSpec)."""
+    if kind == "norm":
+        return 1.0 + 0.1 * z
+    if kind == "around_zero":
+        return 0.1 * z
+    if kind == "unit_interval":
+        return torch.sigmoid(z)
+    if kind == "bias":
+        return z
+    return sigma * z
+
+
 def random_tensors(specs: Mapping[str, TensorSpec], seed: int, sigma: float = 0.02,
                    dtype: torch.dtype = torch.bfloat16) -> Iterator[Tuple[str, torch.Tensor]]:
     """Seeded random weights, one tensor after the other in the order of ``specs``.
@@ -99,11 +112,7 @@ def random_tensors(specs: Mapping[str, TensorSpec], seed: int, sigma: float = 0.
             yield name, torch.randint(0, 2 ** 15, spec.shape, generator=g, dtype=torch.int32)
             continue
         z = torch.randn(spec.shape, generator=g, dtype=torch.float32)
-        if spec.kind == "norm":
-            z = 1.0 + 0.1 * z
-        else:
-            z = sigma * z
-        yield name, z.to(dtype)
+        yield name, shape_values(spec.kind, z, sigma).to(dtype)
 
 
 def write_model_folder(folder: str | Path, config: Mapping[str, object], specs: Mapping[str, TensorSpec],
