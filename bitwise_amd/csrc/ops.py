@@ -649,7 +649,7 @@ def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor
 # ------------------------------------------------------------------------------ mixers with a state per request
 
 RECUR_DECAY_PER_CHANNEL, RECUR_SCALAR_GATES = 0, 1
-RECUR_MAX_DIM = 128          # key channels of a head that the recurrence keeps in a lane's registers
+RECUR_MAX_DIM = 256          # key channels of a head that the recurrence keeps in a lane's registers
 GATE_SIGMOID, GATE_SILU = 0, 1
 ACT_SILU, ACT_GELU_TANH = 0, 1
 

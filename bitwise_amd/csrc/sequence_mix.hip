@@ -240,6 +240,7 @@ int launch_recurrence(const RecurArgs& a, int nseq, hipStream_t s) {
   else if (a.dim <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 32>), grid, block, 0, s, a);
   else if (a.dim <= 64) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 64>), grid, block, 0, s, a);
   else if (a.dim <= 128) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 128>), grid, block, 0, s, a);
+  else if (a.dim <= 256) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 256>), grid, block, 0, s, a);
   else return -4;
   return BW_LAUNCH_CHECK();
 }

@@ -94,8 +94,8 @@ class LatentAttention(Mixer):
         if q.dtype != dkv.dtype:
             raise ValueError("q and dkv projections must be stored in one dtype to be stacked")
         self.q_off, self.dkv_off = 0, q.shape[0]
-        self.proj = Linear(torch.cat([q, dkv], dim=0), self.rt, matrix_cores=self.width % 8 == 0)
-        self.o = Linear(tensors["o"], self.rt, matrix_cores=(self.heads * self.vdim) % 8 == 0)
+        self.proj = Linear(torch.cat([q, dkv], dim=0), self.rt)
+        self.o = Linear(tensors["o"], self.rt)
         dev = self.rt.device
         self.latent_norm = tensors["dkv.norm"].to(dev).float().contiguous()
         self.sink = tensors["sink"].to(dev).float().contiguous()

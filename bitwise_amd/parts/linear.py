@@ -31,9 +31,9 @@ class Linear:
                 raise ValueError(f"a bias of {tuple(bias.shape)} does not fit a weight of {tuple(weight.shape)}")
             self.bias = bias.to(runtime.device).float().contiguous()      # (widening is exact)
         self.out_features, self.in_features = self.weight.shape
-        self.mfma = bool(matrix_cores) and runtime.bf16 and self.weight.dtype == torch.bfloat16
-        if self.mfma and self.in_features % 8:
-            raise ValueError(f"bfloat16 matrix product: inner size {self.in_features} must be a multiple of 8")
+        # (the matrix-core kernels load operands 16 bytes at a time: an inner size that is no multiple of 8 stays on the
+        # 32-bit kernels, which take any)
+        self.mfma = bool(matrix_cores) and runtime.bf16 and self.weight.dtype == torch.bfloat16 and self.in_features % 8 == 0
 
     def nbytes(self) -> int:
         return self.weight.numel() * self.weight.element_size() + (0 if self.bias is None else self.bias.numel() * 4)

@@ -72,8 +72,8 @@ class _MatrixMemoryMixer(Mixer):
             self.offsets[name] = off
             off += n
         self.proj_width = off
-        self.proj = Linear(torch.cat(parts, dim=0), self.rt, matrix_cores=self.width % 8 == 0)
-        self.o = Linear(tensors["o"], self.rt, matrix_cores=(self.heads * self.vdim) % 8 == 0)
+        self.proj = Linear(torch.cat(parts, dim=0), self.rt)
+        self.o = Linear(tensors["o"], self.rt)
         self.norm_weight = tensors["norm"].to(self.rt.device).float().contiguous()
 
     def state_spec(self) -> StateSpec:

@@ -16,6 +16,16 @@ import torch
 F = torch.float64
 
 
+def identity(x):
+    return x
+
+
+def round_bf16(x: torch.Tensor) -> torch.Tensor:
+    """Round to the nearest bfloat16 (ties to even) and come back: the places where the engine's bfloat16 mode hands a
+    value to a matrix product or to the cache."""
+    return x.to(torch.float32).to(torch.bfloat16).to(F)
+
+
 def to64(tensors: Mapping[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
     return {k: v.to(F) for k, v in tensors.items()}
 
@@ -39,11 +49,11 @@ def token_shift(h: torch.Tensor, mix: torch.Tensor) -> torch.Tensor:
     return h + (prev - h) * mix
 
 
-def dense_ff(h, w, pre):
-    return (gelu_tanh(h @ w[pre + "mlp.gate"].T) * (h @ w[pre + "mlp.up"].T)) @ w[pre + "mlp.down"].T
+def dense_ff(h, w, pre, rnd=identity):
+    return rnd(gelu_tanh(h @ w[pre + "mlp.gate"].T) * (h @ w[pre + "mlp.up"].T)) @ w[pre + "mlp.down"].T
 
 
-def mlstm_mixer(h, w, pre, m, eps):
+def mlstm_mixer(h, w, pre, m, eps, rnd=identity):
     H, D, V, cap = m["heads"], m["dim"], m["vdim"], float(m["gate_cap"])
     T = h.shape[0]
     q = (h @ w[pre + "mix.q"].T).view(T, H, D) * D ** -0.5
@@ -67,10 +77,10 @@ def mlstm_mixer(h, w, pre, m, eps):
         out[t] = num / den[:, None]
     o = rms_unit(out, eps).reshape(T, H * V) * w[pre + "mix.norm"]
     o = o * torch.sigmoid(h @ w[pre + "mix.g"].T)
-    return o @ w[pre + "mix.o"].T
+    return rnd(o) @ w[pre + "mix.o"].T
 
 
-def gla_mixer(h, w, pre, m, eps):
+def gla_mixer(h, w, pre, m, eps, rnd=identity):
     H, D, V, tau = m["heads"], m["dim"], m["vdim"], float(m["tau"])
     T = h.shape[0]
     q = (h @ w[pre + "mix.q"].T).view(T, H, D) * D ** -0.5
@@ -85,7 +95,7 @@ def gla_mixer(h, w, pre, m, eps):
         out[t] = torch.einsum("hdv,hd->hv", S, q[t])
     o = (rms_unit(out, eps) * w[pre + "mix.norm"]).reshape(T, H * V)
     o = o * torch.nn.functional.silu(h @ w[pre + "mix.g"].T)
-    return o @ w[pre + "mix.o"].T
+    return rnd(o) @ w[pre + "mix.o"].T
 
 
 def rotate_half(x: torch.Tensor, positions: torch.Tensor, base: float, dims: int) -> torch.Tensor:
@@ -99,16 +109,16 @@ def rotate_half(x: torch.Tensor, positions: torch.Tensor, base: float, dims: int
     return torch.cat([u * torch.cos(a) - v * torch.sin(a), v * torch.cos(a) + u * torch.sin(a), x[..., dims:]], -1)
 
 
-def latent_attention_mixer(h, w, pre, m, eps):
+def latent_attention_mixer(h, w, pre, m, eps, rnd=identity):
     H, D, R, V, C = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
-    base, scale = float(m["rot"]["base"]), float(m["scale"])
+    base, dims, scale = float(m["rot"]["base"]), int(m["rot"]["dims"]), float(m["scale"])
     T = h.shape[0]
     pos = torch.arange(T)
     q = (h @ w[pre + "mix.q"].T).view(T, H, D + R)
-    q_plain, q_rot = q[..., :D], rotate_half(q[..., D:], pos, base, R)
+    q_plain, q_rot = q[..., :D], rotate_half(q[..., D:], pos, base, dims)
     dkv = h @ w[pre + "mix.dkv"].T
-    c = rms_unit(dkv[:, :C], eps) * w[pre + "mix.dkv.norm"]
-    k_rot = rotate_half(dkv[:, C:], pos, base, R)                      # one for all heads
+    c = rnd(rms_unit(dkv[:, :C], eps) * w[pre + "mix.dkv.norm"])          # what the cache holds
+    k_rot = rnd(rotate_half(dkv[:, C:], pos, base, dims))                  # one for all heads
     k_plain = (c @ w[pre + "mix.uk"].T).view(T, H, D)
     val = (c @ w[pre + "mix.uv"].T).view(T, H, V)
     out = torch.zeros(T, H, V, dtype=F)
@@ -119,27 +129,51 @@ def latent_attention_mixer(h, w, pre, m, eps):
         e = torch.exp(s - top[:, None])
         den = e.sum(-1) + torch.exp(sink - top)
         out[t] = torch.einsum("hj,jhv->hv", e / den[:, None], val[:t + 1])
-    return out.reshape(T, H * V) @ w[pre + "mix.o"].T
+    return rnd(out.reshape(T, H * V)) @ w[pre + "mix.o"].T
 
 
 MIXERS = {"mlstm": mlstm_mixer, "gla": gla_mixer, "latent_attention": latent_attention_mixer}
 
 
-def layer(x, w, i, spec, eps):
+def layer(x, w, i, spec, eps, rnd=identity):
     pre = f"l{i}."
-    h = token_shift(norm_around_zero(x, w[pre + "norm1"], eps), w[pre + "shift"])
-    y = MIXERS[spec["type"]](h, w, pre, spec["mixer"], eps)
+    h = rnd(token_shift(norm_around_zero(x, w[pre + "norm1"], eps), w[pre + "shift"]))
+    y = MIXERS[spec["type"]](h, w, pre, spec["mixer"], eps, rnd)
     if spec.get("mlp") is not None:
-        y = y + dense_ff(norm_around_zero(x, w[pre + "norm2"], eps), w, pre)
+        y = y + dense_ff(rnd(norm_around_zero(x, w[pre + "norm2"], eps)), w, pre, rnd)
     return x + y
 
 
-def forward(config: Mapping, w: Mapping[str, torch.Tensor], tokens: List[int], keep_layers: Optional[list] = None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence (float64)."""
+def forward(config: Mapping, w: Mapping[str, torch.Tensor], tokens: List[int], keep_layers: Optional[list] = None,
+            rnd=identity) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence (float64).  ``rnd`` = round_bf16 rounds where the engine's bfloat16 mode does:
+    the inputs of the projections, the feed-forward's gated unit, what the mixers hand to their output projection,
+    what the cache holds; every sum, state, gate, score and norm stays exact."""
     eps = float(config["norm"]["eps"])
     x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)]
     for i, spec in enumerate(config["layers"]):
-        x = layer(x, w, i, spec, eps)
+        x = layer(x, w, i, spec, eps, rnd)
         if keep_layers is not None:
             keep_layers.append(x.clone())
-    return norm_around_zero(x, w["final.norm"], eps) @ w["head"].T
+    return rnd(norm_around_zero(x, w["final.norm"], eps)) @ w["head"].T
+
+
+def generate_greedy(config: Mapping, w: Mapping[str, torch.Tensor], prompt: List[int], new_tokens: int) -> List[int]:
+    """Greedy continuation, the whole sequence recomputed for every token (the first maximum wins)."""
+    toks, out = list(prompt), []
+    for _ in range(new_tokens):
+        nxt = int(torch.argmax(forward(config, w, toks)[-1]))
+        out.append(nxt)
+        toks.append(nxt)
+    return out
+
+
+def logits_error(got, want, quantile: float = 1.0) -> float:
+    """A row's error: the root mean square of the difference (its mean taken off) over that of the wanted row; the
+    largest over the rows, or the given quantile of them."""
+    import numpy as np
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    ref = want - want.mean(-1, keepdims=True)
+    return float(np.quantile(np.sqrt((d * d).mean(-1)) / np.sqrt((ref * ref).mean(-1)), quantile))
