@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep] [--kuponex]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -44,6 +44,57 @@ LLAMA3_8B = {
     "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 8192,
     "bos_token_id": 1, "eos_token_id": 2,
 }
+
+
+def kuponex_shape(width: int, ff: int, groups: int, vocab: int = 32000) -> dict:
+    """A Kuponex of ``groups`` x (attention over a compressed cache, matrix LSTM, two layers of gated linear attention)
+    with head sizes that grow with the width as real layers' do."""
+    big = width >= 4096
+    heads = width // 128
+    layers = []
+    for _ in range(groups):
+        layers.append({"type": "latent_attention", "mlp": {"kind": "dense", "ff": ff},
+                       "mixer": {"heads": heads, "dim": 128 if big else 96, "rot_dim": 64 if big else 32, "vdim": 128,
+                                 "kv_rank": 512 if big else 256, "scale": (192 if big else 128) ** -0.5,
+                                 "rot": {"base": 500000.0, "dims": 64 if big else 32}}})
+        layers.append({"type": "mlstm", "mlp": {"kind": "dense", "ff": ff},
+                       "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "gate_cap": 15.0}})
+        for _ in range(2):
+            layers.append({"type": "gla", "mlp": {"kind": "dense", "ff": ff},
+                           "mixer": {"heads": heads, "dim": 64, "vdim": 128, "tau": 16.0, "rank": 64}})
+    return {"architecture": "Kuponex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": layers,
+            "max_positions": 16384, "eos_token_id": 2}
+
+
+def llama_shape(width: int, ff: int, layers: int, vocab: int = 32000) -> dict:
+    """The Llama decoder of the same width, depth, feed-forward and vocabulary (heads of 128, a quarter as many kv heads)."""
+    return {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu", "vocab_size": vocab,
+            "hidden_size": width, "num_hidden_layers": layers, "num_attention_heads": width // 128,
+            "num_key_value_heads": max(1, width // 512), "head_dim": 128, "intermediate_size": ff, "rope_theta": 500000.0,
+            "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "max_position_embeddings": 16384, "bos_token_id": 1, "eos_token_id": 2}
+
+
+def kuponex_comparison(bw, torch, steps: int, dtype: str, only: str = "") -> int:
+    """Prefill and decode of Kuponex at two layer sizes beside the Llama decoder of equal width, depth and feed-forward:
+    one JSON object a line."""
+    from bitwise_amd.measure import PEAK_FLOPS, measure_decode, measure_prefill
+    for name, width, ff, groups in (("2048x8192", 2048, 8192, 2), ("4096x14336", 4096, 14336, 2)):
+        for arch, cfg in (("Kuponex", kuponex_shape(width, ff, groups)), ("Llama", llama_shape(width, ff, 4 * groups))):
+            if only and only.lower() != arch.lower():
+                continue
+            model = bw.Model.random(cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
+            for tokens in (512, 2048):
+                m = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[dtype], tokens)
+                print(json.dumps({"shape": name, "model": arch, "dtype": dtype, "prefill_tokens": tokens, "ms": m["ms"],
+                                  "tok_s": m["value"], "frac_of_matrix_peak": m["frac"]}), flush=True)
+            for batch in (1, 8, 64):
+                m = measure_decode(bw, torch, model, cfg, dtype, batch, steps, 4, context=2048)
+                print(json.dumps({"shape": name, "model": arch, "dtype": dtype, "decode_batch": batch, "context": 2048,
+                                  "ms_per_step": m["ms_per_step"], "tok_s": m["tok_s"], "frac_of_8_TBs": m["roofline"]["frac"]}),
+                      flush=True)
+            del model
+            torch.cuda.empty_cache()
+    return 0
 
 
 def sweep(bw, torch, steps: int, dtype: str) -> int:
@@ -95,6 +146,9 @@ def main() -> int:
     ap.add_argument("--sweep", action="store_true",
                     help="print a table instead of the line: decode at batches 1 to 128 and contexts of 512 to 8,192 tokens, prefills "
                          "of 128 to 2,048 tokens, at both shapes (with --dtype fp32: a coarser grid at the small shape)")
+    ap.add_argument("--kuponex", nargs="?", const="both", default="", choices=["both", "kuponex", "llama"],
+                    help="print a table instead of the line: prefill and decode of the Kuponex design at two layer sizes beside "
+                         "the Llama decoder of equal width, depth and feed-forward (or only one of the two)")
     ap.add_argument("--no-points", action="store_true",
                     help="only the headline: skip decode at batch 1 and 64, the 32-bit path and the Llama-3-8B sizes")
     args = ap.parse_args()
@@ -110,6 +164,8 @@ def main() -> int:
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     if args.sweep:
         return sweep(bw, torch, args.steps, dtype)
+    if args.kuponex:
+        return kuponex_comparison(bw, torch, min(args.steps, 32), dtype, "" if args.kuponex == "both" else args.kuponex)
     if args.mixed:
         from bitwise_amd.measure import measure_prefill_beside_decodes, measure_qkv_row_orders
         cfg = dict(SMOLLM2_1_7B if args.shape == "smollm2" else LLAMA3_8B, max_position_embeddings=16384)

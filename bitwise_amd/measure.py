@@ -12,7 +12,37 @@ PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12, "bfloat16": 2.5e15, "float32": 157.3e12}
 
 
+def vocab_of(cfg: dict) -> int:
+    return int(cfg["vocab_size"] if "vocab_size" in cfg else cfg["vocab"])
+
+
+def kuponex_prefill_flops(cfg: dict, tokens: int) -> float:
+    """Multiply-adds times two of one prompt: every projection, the feed-forward, the recurrences' state updates and
+    read-outs, and the attention over the compressed cache in the cache's own space (scores and weighted sums over
+    kv_rank + rot_dim and kv_rank elements per key and head, the projections into and out of that space)."""
+    w, total = cfg["width"], 0.0
+    for layer in cfg["layers"]:
+        m, per_token, quadratic = layer["mixer"], 0.0, 0.0
+        H, D, V = m["heads"], m["dim"], m["vdim"]
+        if layer["type"] == "latent_attention":
+            R, C = m["rot_dim"], m["kv_rank"]
+            per_token = w * (H * (D + R) + C + R) + H * D * C + H * C * V + H * V * w
+            quadratic = H * (2 * C + R) * tokens * (tokens + 1) / 2
+        else:
+            inner = H * (2 * D + 2 * V)
+            inner += (2 * H) if layer["type"] == "mlstm" else (m["rank"] + 0)
+            per_token = w * inner + H * V * w + 2 * H * D * V
+            if layer["type"] == "gla":
+                per_token += m["rank"] * H * D
+        if layer.get("mlp"):
+            per_token += 3 * w * layer["mlp"]["ff"]
+        total += 2 * (per_token * tokens + quadratic)
+    return total + 2 * w * cfg["vocab"]
+
+
 def prefill_flops(cfg: dict, tokens: int) -> float:
+    if cfg.get("architecture") == "Kuponex":
+        return kuponex_prefill_flops(cfg, tokens)
     h, inter, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     qd = cfg["num_attention_heads"] * cfg["head_dim"]
     kvd = cfg["num_key_value_heads"] * cfg["head_dim"]
@@ -63,7 +93,7 @@ def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float, 
     g = torch.Generator().manual_seed(99)
     times = []
     for _ in range(8):
-        prompt = torch.randint(0, cfg["vocab_size"], (tokens,), generator=g).tolist()
+        prompt = torch.randint(0, vocab_of(cfg), (tokens,), generator=g).tolist()
         engine.add_request(prompt, bw.SamplingParams(max_new_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -91,7 +121,7 @@ def measure_chunked_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops:
     g = torch.Generator().manual_seed(98)
     times, steps = [], 0
     for _ in range(4):
-        prompt = torch.randint(0, cfg["vocab_size"], (tokens,), generator=g).tolist()
+        prompt = torch.randint(0, vocab_of(cfg), (tokens,), generator=g).tolist()
         engine.add_request(prompt, bw.SamplingParams(max_new_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -120,13 +150,13 @@ def measure_prefill_beside_decodes(bw, torch, model, cfg: dict, dtype: str, toke
     engine = bw.Engine(model, None, ecfg)
     g = torch.Generator().manual_seed(97)
     for _ in range(decoders):
-        prompt = torch.randint(0, cfg["vocab_size"], (512,), generator=g).tolist()
+        prompt = torch.randint(0, vocab_of(cfg), (512,), generator=g).tolist()
         engine.add_request(prompt, bw.SamplingParams(max_new_tokens=400, ignore_eos=True))
     while engine.num_waiting or any(s.computed < s.prompt_len for s in engine.sched.running):
         engine.step()
     times, steps = [], 0
     for _ in range(4):
-        prompt = torch.randint(0, cfg["vocab_size"], (tokens,), generator=g).tolist()
+        prompt = torch.randint(0, vocab_of(cfg), (tokens,), generator=g).tolist()
         rid = engine.add_request(prompt, bw.SamplingParams(max_new_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -202,17 +232,20 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
     fill_steps = -(-batch * context // (2048 - batch - 64)) + 1
     new_tokens = steps + warmup + fill_steps + 8
     eng = make_engine(bw, model, batch, new_tokens, dtype, context, decode_phases, portion_align)
-    fill(eng, bw, torch, batch, cfg["vocab_size"], new_tokens, seed=batch, context=context)
+    fill(eng, bw, torch, batch, vocab_of(cfg), new_tokens, seed=batch, context=context)
     assert len(eng.sched.running) == batch
     secs = time_decode(eng, torch, steps, warmup)
     assert len(eng.sched.running) == batch, "a request finished inside the timed steps"
     kv_token = eng.exec.storage.bytes_per_token()
-    del eng
+    # state that a request keeps in a slot is read and written once a step
+    storage = eng.exec.storage
+    slot_bytes = sum(t[0].numel() * t.element_size() for t in list(storage.states.values()) + list(storage.block_states.values()))
+    del eng, storage
     ms = secs / steps * 1e3
     # keys a decoded token reads, on average: the prompt, what the request decoded while later
     # prompts were prefilled, the warm-up, and half the timed steps
     avg_ctx = context + batch * context / 2048 * (batch - 1) / (2 * batch) + warmup + (steps + 1) / 2
-    step_bytes = model.weight_bytes + batch * avg_ctx * kv_token
+    step_bytes = model.weight_bytes + batch * avg_ctx * kv_token + 2 * batch * slot_bytes
     achieved = step_bytes / (ms * 1e-3) / 1e9
     return {"tok_s": round(batch * steps / secs, 1), "ms_per_step": round(ms, 4),
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -229,7 +262,7 @@ def measure_serving(bw, torch, model, cfg: dict, dtype: str, requests: int = 64,
     work = []
     for _ in range(requests):
         n, new = rng.randint(128, 2048), rng.randint(64, 512)
-        work.append((torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist(), new))
+        work.append((torch.randint(0, vocab_of(cfg), (n,), generator=g).tolist(), new))
     block = 16
     pages = sum((len(p) + new + 2 * block) // block + 1 for p, new in work)
     ecfg = bw.EngineConfig(num_blocks=pages, max_batched_tokens=2048, max_num_seqs=requests, prefix_caching=False,

@@ -1,6 +1,6 @@
 """The Kuponex decoder as a ModelSpec: parallel layers x += mixer(shift(norm1(x))) + ff(norm2(x)) whose mixers are,
-layer by layer, a matrix LSTM, gated linear attention or attention over a compressed cache; norms with weights
-stored around zero; a gated GELU feed-forward; a final norm and an untied head.  Layer i's tensors start with
+layer by layer, a matrix LSTM, gated linear attention or attention over a compressed cache; norms whose weights
+are kept as their distance from 1; a gated GELU feed-forward; a final norm and an untied head.  Layer i's tensors start with
 ``l<i>.``: norm1, norm2, shift, mix.*, mlp.{gate,up,down}; the rest are ``embed``, ``final.norm`` and ``head``."""
 
 from __future__ import annotations

@@ -14,7 +14,7 @@ from .base import Norm, StateSpec, TensorSpec, register_norm
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
     """params: width, eps; optional ``offset`` (the stored weight w is applied as offset + w; 0 by default, 1 for a
-    weight stored around zero) and ``tensor`` (the weight's name behind the prefix, "weight" by default).
+    weight kept as its distance from 1) and ``tensor`` (the weight's name behind the prefix, "weight" by default).
     The sum of squares, the root and both products are 32-bit; the output has the mode's activation dtype."""
 
     graph_safe = True
