@@ -51,7 +51,7 @@ struct PrepArgs {
 // A workgroup a row.  The rotated part: elements i and i + rotary/2 (i < rotary/2) are a pair; elements from
 // ``rotary`` on pass unchanged.
 template <typename CT>
-__global__ __launch_bounds__(256) void latent_prep_kernel(PrepArgs a, CT* __restrict__ cache) {
+__global__ __launch_bounds__(256) void latent_prep_kernel(PrepArgs a, CT* __restrict__ cache, CT* __restrict__ latent_t) {
   const int row = blockIdx.x;
   const int pos = a.positions[row];
   if (pos < 0) return;
@@ -70,6 +70,10 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(PrepArgs a, CT* __rest
     const int page = a.block_table[(size_t)a.row_seq[row] * a.table_stride + pos / a.page_size];
     CT* dst = cache + ((size_t)page * a.page_size + pos % a.page_size) * width;
     for (int i = threadIdx.x; i < a.rank; i += blockDim.x) store_f(dst + i, (dkv[i] * inv) * a.norm_w[i]);
+    if (latent_t != nullptr) {      // the latent once more, transposed within its page: [page][element][slot]
+      CT* tp = latent_t + (size_t)page * a.rank * a.page_size + pos % a.page_size;
+      for (int i = threadIdx.x; i < a.rank; i += blockDim.x) store_f(tp + (size_t)i * a.page_size, (dkv[i] * inv) * a.norm_w[i]);
+    }
     const float* kr = dkv + a.rank;
     for (int i = threadIdx.x; i < a.rot; i += blockDim.x) {
       float v;
@@ -318,12 +322,255 @@ int launch_shared_key(const SharedKeyArgs& a, const CT* cache, int num_tiles, hi
   return -8;
 }
 
+
+// ------------------------------------------------------------------------- the same attention on the matrix cores
+
+// bfloat16 caches whose key vectors are whole 16-byte groups.  A wave per (tile, group of heads, split of the keys): 16
+// query vectors (16 / hg rows x hg heads), keys in blocks of 64.  Scores: v_mfma_f32_16x16x32_bf16 with the keys as rows
+// (operand A, straight from the cache: a lane reads 8 consecutive elements of its key) and the queries as columns
+// (operand B, rounded to bfloat16 once, from LDS); 32-bit sums, scaled, masked, softmax in 32-bit with a running maximum.
+// The weighted sum takes the weights rounded to bfloat16 as columns and the values as rows d of a second copy of the
+// latent that the cache write leaves transposed, [page][d][slot]: a lane's 8 keys are two runs of 4 consecutive slots
+// (the keys of its four scores in two neighbouring sub-blocks of 16).  A lane's scores, sums and outputs all belong to
+// query (lane mod 16).  With nsplit > 1 a wave takes kchunk keys and leaves (maximum, denominator, sums) for
+// shared_key_combine_kernel; the sink joins where the result is finished.
+struct MfmaAttnArgs {
+  const float* q;
+  int ldq;
+  const int32_t* positions;
+  const int32_t* block_table;
+  int table_stride;
+  const int32_t* tiles;
+  const float* sink;
+  float* out;
+  int ldo;
+  float* partial;          // [tiles][heads][nsplit][dv + 2]
+  int heads, dk, dv, page_size, window, hg, num_pages, nsplit, kchunk;
+  float scale;
+};
+
+__device__ __forceinline__ float across_groups_max(float v) {
+  float a, b;
+  lane_halves<32>(v, a, b);
+  v = fmaxf(a, b);
+  lane_halves<16>(v, a, b);
+  return fmaxf(a, b);
+}
+
+__device__ __forceinline__ float across_groups_sum(float v) {
+  float a, b;
+  lane_halves<32>(v, a, b);
+  v = a + b;
+  lane_halves<16>(v, a, b);
+  return a + b;
+}
+
+template <int NDT>
+__global__ __launch_bounds__(64) void shared_key_attention_mfma_kernel(MfmaAttnArgs a, const bf16_t* __restrict__ kc,
+                                                                       const bf16_t* __restrict__ vt) {
+  extern __shared__ bf16_t qs[];           // [16][qstride]
+  const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+  const int t = blockIdx.x, h0 = blockIdx.y * a.hg, split = blockIdx.z;
+  int r0, nr, seq;
+  if (a.tiles != nullptr) {
+    r0 = a.tiles[4 * t];
+    nr = a.tiles[4 * t + 1];
+    seq = a.tiles[4 * t + 2];
+  } else {
+    r0 = t;
+    nr = 1;
+    seq = t;
+  }
+  if (nr <= 0) return;
+  const int pos0 = a.positions[r0];
+  if (pos0 < 0) return;
+  const int pmax = pos0 + nr - 1;
+  const int rl = n / a.hg, h = h0 + n % a.hg;
+  const bool qok = rl < nr && h < a.heads;
+  const int qpos = qok ? pos0 + rl : -1;
+  const int qlo = a.window > 0 ? max(0, qpos - a.window + 1) : 0;
+  const int dkp = (a.dk + 31) & ~31, qstride = dkp + 8;
+  for (int e = lane; e < 16 * dkp; e += 64) {
+    const int qn = e / dkp, d = e % dkp;
+    const int r2 = qn / a.hg, h2 = h0 + qn % a.hg;
+    const float v = (r2 < nr && h2 < a.heads && d < a.dk) ? a.q[(size_t)(r0 + r2) * a.ldq + h2 * a.dk + d] : 0.0f;
+    qs[qn * qstride + d] = f32_to_bf16(v);
+  }
+  __syncthreads();
+
+  const int lo_first = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
+  int k_begin = lo_first & ~63, k_end = pmax + 1;
+  if (a.nsplit > 1) {
+    k_begin = max(k_begin, split * a.kchunk);
+    k_end = min(k_end, (split + 1) * a.kchunk);
+  }
+  const int32_t* table = a.block_table + (size_t)seq * a.table_stride;
+  const int ps = a.page_size, dk = a.dk, dv = a.dv;
+
+  float m = -INFINITY, lsum = 0.0f;
+  f32x4 acc[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) acc[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  for (int kb0 = k_begin; kb0 < k_end; kb0 += 64) {
+    const bf16_t* krow[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int kj = min(kb0 + 16 * u + n, pmax);
+      const int page = min(max(table[kj / ps], 0), a.num_pages - 1);
+      krow[u] = kc + ((size_t)page * ps + kj % ps) * dk;
+    }
+    f32x4 st[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) st[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int d0 = 8 * g; d0 < dkp; d0 += 32) {
+      const u32x4 qf = *reinterpret_cast<const u32x4*>(qs + n * qstride + d0);
+      u32x4 kf[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) kf[u] = d0 < dk ? *reinterpret_cast<const u32x4*>(krow[u] + d0) : (u32x4){0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u]), as_bf16x8(qf), st[u], 0, 0, 0);
+    }
+    // this lane: query n, keys kb0 + 16u + 4g + i
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb0 + 16 * u + 4 * g + i;
+        const bool valid = key <= qpos && key >= qlo && key < k_end;
+        const float sv = valid ? st[u][i] * a.scale : -INFINITY;
+        st[u][i] = sv;
+        mx = fmaxf(mx, sv);
+      }
+    mx = across_groups_max(mx);
+    const float mn = fmaxf(m, mx);
+    const float base = mn == -INFINITY ? 0.0f : mn;
+    const float corr = m == -INFINITY ? 0.0f : fast_exp(m - base);
+    float psum = 0.0f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = st[u][i] == -INFINITY ? 0.0f : fast_exp(st[u][i] - base);
+        st[u][i] = pv;
+        psum += pv;
+      }
+    lsum = lsum * corr + psum;
+    m = mn;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) acc[dt] *= corr;
+    const bool ragged = kb0 + 63 > pmax || kb0 < lo_first;       // slots behind the last key, or before the window, may hold anything
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const u32x4 pf = {pack_bf16x2(st[2 * w][0], st[2 * w][1]), pack_bf16x2(st[2 * w][2], st[2 * w][3]),
+                        pack_bf16x2(st[2 * w + 1][0], st[2 * w + 1][1]), pack_bf16x2(st[2 * w + 1][2], st[2 * w + 1][3])};
+      const int key0 = kb0 + 32 * w + 4 * g, key1 = key0 + 16;
+      const int c0 = min(key0, pmax & ~3), c1 = min(key1, pmax & ~3);
+      const bf16_t* b0 = vt + (size_t)min(max(table[c0 / ps], 0), a.num_pages - 1) * dv * ps + c0 % ps;
+      const bf16_t* b1 = vt + (size_t)min(max(table[c1 / ps], 0), a.num_pages - 1) * dv * ps + c1 % ps;
+      uint32_t keep0[2] = {0xffffffffu, 0xffffffffu}, keep1[2] = {0xffffffffu, 0xffffffffu};
+      if (ragged) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t bits = 0xffffu << (16 * (e & 1));
+          if (key0 + e > pmax || key0 + e < lo_first) keep0[e >> 1] &= ~bits;
+          if (key1 + e > pmax || key1 + e < lo_first) keep1[e >> 1] &= ~bits;
+        }
+      }
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        const int d = 16 * dt + n;
+        u32x4 vf = {0u, 0u, 0u, 0u};
+        if (d < dv) {
+          const u32x2 x0 = *reinterpret_cast<const u32x2*>(b0 + (size_t)d * ps);
+          const u32x2 x1 = *reinterpret_cast<const u32x2*>(b1 + (size_t)d * ps);
+          vf = (u32x4){x0[0] & keep0[0], x0[1] & keep0[1], x1[0] & keep1[0], x1[1] & keep1[1]};
+        }
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf), as_bf16x8(pf), acc[dt], 0, 0, 0);
+      }
+    }
+  }
+  lsum = across_groups_sum(lsum);
+  if (!qok) return;
+  if (a.nsplit > 1) {
+    float* part = a.partial + (((size_t)t * a.heads + h) * a.nsplit + split) * (dv + 2);
+    if (g == 0) {
+      part[0] = m;
+      part[1] = lsum;
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = 16 * dt + 4 * g + i;
+        if (d < dv) part[2 + d] = acc[dt][i];
+      }
+    return;
+  }
+  const float sk = a.sink != nullptr ? a.sink[h] : -INFINITY;
+  const float mf = fmaxf(m, sk);
+  const float cm = m == -INFINITY ? 0.0f : fast_exp(m - mf);
+  const float lt = lsum * cm + (sk == -INFINITY ? 0.0f : fast_exp(sk - mf));
+  const float w = lt > 0.0f ? cm / lt : 0.0f;
+  float* orow = a.out + (size_t)(r0 + rl) * a.ldo + h * dv;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = 16 * dt + 4 * g + i;
+      if (d < dv) orow[d] = acc[dt][i] * w;
+    }
+}
+
+// The splits of one (single-row tile, head) joined: the largest maximum (the sink's score among them), every split's
+// denominator and sums scaled to it, in split order.
+__global__ __launch_bounds__(64) void shared_key_combine_kernel(MfmaAttnArgs a) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int r0 = a.tiles != nullptr ? a.tiles[4 * t] : t;
+  if (a.tiles != nullptr && a.tiles[4 * t + 1] <= 0) return;
+  if (a.positions[r0] < 0) return;
+  const float* part = a.partial + ((size_t)t * a.heads + h) * a.nsplit * (a.dv + 2);
+  const int live = min(a.nsplit, a.positions[r0] / a.kchunk + 1);      // splits beyond the row's position hold nothing
+  const float sk = a.sink != nullptr ? a.sink[h] : -INFINITY;
+  float mt = sk;
+  for (int s = 0; s < live; ++s) mt = fmaxf(mt, part[(size_t)s * (a.dv + 2)]);
+  float lt = sk == -INFINITY ? 0.0f : fast_exp(sk - mt);
+  for (int s = 0; s < live; ++s) {
+    const float ms = part[(size_t)s * (a.dv + 2)];
+    if (ms != -INFINITY) lt += part[(size_t)s * (a.dv + 2) + 1] * fast_exp(ms - mt);
+  }
+  const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
+  for (int d = threadIdx.x; d < a.dv; d += 64) {
+    float o = 0.0f;
+    for (int s = 0; s < live; ++s) {
+      const float ms = part[(size_t)s * (a.dv + 2)];
+      if (ms != -INFINITY) o = fmaf(part[(size_t)s * (a.dv + 2) + 2 + d], fast_exp(ms - mt), o);
+    }
+    a.out[(size_t)r0 * a.ldo + h * a.dv + d] = o * inv;
+  }
+}
+
+int launch_shared_key_mfma(const MfmaAttnArgs& a, const bf16_t* kc, const bf16_t* vt, int num_tiles, hipStream_t s) {
+  const int dkp = (a.dk + 31) & ~31;
+  const size_t bytes = (size_t)16 * (dkp + 8) * sizeof(bf16_t);
+  const dim3 grid(num_tiles, (a.heads + a.hg - 1) / a.hg, a.nsplit), block(64);
+  const int ndt = (a.dv + 15) / 16;
+  if (ndt <= 4) hipLaunchKernelGGL(shared_key_attention_mfma_kernel<4>, grid, block, bytes, s, a, kc, vt);
+  else if (ndt <= 8) hipLaunchKernelGGL(shared_key_attention_mfma_kernel<8>, grid, block, bytes, s, a, kc, vt);
+  else if (ndt <= 16) hipLaunchKernelGGL(shared_key_attention_mfma_kernel<16>, grid, block, bytes, s, a, kc, vt);
+  else if (ndt <= 32) hipLaunchKernelGGL(shared_key_attention_mfma_kernel<32>, grid, block, bytes, s, a, kc, vt);
+  else return -4;
+  if (a.nsplit > 1) hipLaunchKernelGGL(shared_key_combine_kernel, dim3(num_tiles, a.heads), dim3(64), 0, s, a);
+  return BW_LAUNCH_CHECK();
+}
+
 }  // namespace
 
 extern "C" int bw_latent_prep(const float* proj, int ldp, int q_off, int dkv_off, const float* norm_w, float eps,
                               const float* cos_table, const float* sin_table, const int32_t* positions,
                               const int32_t* row_seq, const int32_t* block_table, int table_stride, void* cache,
-                              int cache_is_bf16, float* qa, int ldqa, int rows, int heads, int dim, int rot, int rotary,
+                              void* latent_t, int cache_is_bf16, float* qa, int ldqa, int rows, int heads, int dim, int rot, int rotary,
                               int rank, int page_size, int write_cache, void* stream) {
   if (rows <= 0) return 0;
   if (heads <= 0 || dim < 0 || rot < 0 || rotary < 0 || rotary > rot || (rotary & 1) || rank <= 0 || page_size <= 0) return -2;
@@ -331,8 +578,8 @@ extern "C" int bw_latent_prep(const float* proj, int ldp, int q_off, int dkv_off
   PrepArgs a{proj, ldp, q_off, dkv_off, norm_w, eps, cos_table, sin_table, positions, row_seq, block_table, table_stride,
              qa, ldqa, heads, dim, rot, rotary, rank, page_size, write_cache};
   hipStream_t s = (hipStream_t)stream;
-  if (cache_is_bf16) hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, a, (bf16_t*)cache);
-  else hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(rows), dim3(256), 0, s, a, (float*)cache);
+  if (cache_is_bf16) hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, a, (bf16_t*)cache, (bf16_t*)latent_t);
+  else hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(rows), dim3(256), 0, s, a, (float*)cache, (float*)latent_t);
   return BW_LAUNCH_CHECK();
 }
 
@@ -375,4 +622,27 @@ extern "C" int bw_shared_key_attention(const float* q, int ldq, const int32_t* p
   hipStream_t s = (hipStream_t)stream;
   if (cache_is_bf16) return launch_shared_key<bf16_t>(a, (const bf16_t*)cache, num_tiles, s);
   return launch_shared_key<float>(a, (const float*)cache, num_tiles, s);
+}
+
+// The matrix-core route: bfloat16 cache with key vectors of a multiple of 8 elements, pages of a multiple of 4 slots, and the
+// transposed latents beside it.  nsplit > 1 (single-row tiles, 16 heads a group): every wave takes kchunk keys (a multiple
+// of 64) and ``partial`` holds tiles * heads * nsplit * (dv + 2) floats.
+extern "C" int bw_shared_key_attention_mfma(const float* q, int ldq, const int32_t* positions, const int32_t* block_table,
+                                            int table_stride, const int32_t* tiles, int num_tiles, const void* cache,
+                                            const void* latent_t, int num_pages, const float* sink, float* out, int ldo,
+                                            int heads, int dk, int dv, int page_size, int window, float scale,
+                                            int heads_per_group, int nsplit, int kchunk, float* partial,
+                                            long long partial_floats, void* stream) {
+  if (num_tiles <= 0) return 0;
+  if (heads <= 0 || dk <= 0 || (dk % 8) || dv <= 0 || dv > dk || dv > 512 || page_size < 4 || (page_size % 4) || num_pages <= 0) return -2;
+  if (heads_per_group < 1 || heads_per_group > 16 || (16 % heads_per_group)) return -2;
+  if (ldq < heads * dk || ldo < heads * dv || nsplit < 1) return -2;
+  if (nsplit > 1) {
+    if (heads_per_group != 16 || kchunk < 64 || (kchunk % 64) || partial == nullptr) return -2;
+    if (partial_floats < (long long)num_tiles * heads * nsplit * (dv + 2)) return -6;
+  }
+  if ((reinterpret_cast<uintptr_t>(cache) & 15) || (reinterpret_cast<uintptr_t>(latent_t) & 7)) return -3;
+  MfmaAttnArgs a{q, ldq, positions, block_table, table_stride, tiles, sink, out, ldo, partial, heads, dk, dv, page_size, window,
+                 heads_per_group, num_pages, nsplit, kchunk, scale};
+  return launch_shared_key_mfma(a, (const bf16_t*)cache, (const bf16_t*)latent_t, num_tiles, (hipStream_t)stream);
 }

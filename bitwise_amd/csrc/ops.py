@@ -84,8 +84,11 @@ _SIGS = {
     "bw_head_norm_gate": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int,
                           c_int, c_int, c_float, c_void_p],
     "bw_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_shared_key_attention_mfma": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                     c_void_p, c_longlong, c_void_p],
     "bw_latent_prep": [c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                       c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                       c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                        c_void_p],
     "bw_headwise_linear": [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
                            c_int, c_void_p],
@@ -755,10 +758,11 @@ def glu(gate_up: torch.Tensor, out: torch.Tensor, rows: int, act: int) -> None:
 def latent_prep(proj: torch.Tensor, q_off: int, dkv_off: int, norm_w: torch.Tensor, eps: float, cos: torch.Tensor,
                 sin: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
                 cache: torch.Tensor, qa: torch.Tensor, rows: int, heads: int, dim: int, rot: int, rotary: int, rank: int,
-                page_size: int, write_cache: bool = True) -> None:
+                page_size: int, write_cache: bool = True, latent_t: Optional[torch.Tensor] = None) -> None:
     """From the stacked projections: the latent (RMS-normed) and the rotated shared key part into the row's page slot
     ([pages, page_size * (rank + rot)]), and every head's rotated query part into ``qa`` [rows, heads * (rank + rot)]
-    behind the place of its latent-space part."""
+    behind the place of its latent-space part.  ``latent_t`` [pages, rank * page_size]: the latent once more, transposed
+    within its page ([element][slot]), for the matrix-core attention."""
     _need(proj, torch.float32, "proj")
     _need(norm_w, torch.float32, "norm weight")
     _need(cos, torch.float32, "cos table")
@@ -775,9 +779,13 @@ def latent_prep(proj: torch.Tensor, q_off: int, dkv_off: int, norm_w: torch.Tens
         raise ValueError("latent_prep: cache pages or qa do not fit")
     if min(proj.shape[0], qa.shape[0], positions.numel(), row_seq.numel()) < rows:
         raise ValueError("latent_prep: buffers shorter than the rows")
+    if latent_t is not None and (latent_t.dtype != cache.dtype or latent_t.dim() != 2 or latent_t.shape != (cache.shape[0], page_size * rank)
+                                 or not latent_t.is_contiguous()):
+        raise ValueError("latent_prep: the transposed latents must be [pages, rank * page_size] of the cache's dtype")
     _check(_fn("bw_latent_prep")(proj.data_ptr(), proj.stride(0), q_off, dkv_off, norm_w.data_ptr(), float(eps), cos.data_ptr(),
                                  sin.data_ptr(), positions.data_ptr(), row_seq.data_ptr(), block_table.data_ptr(),
-                                 block_table.stride(0), cache.data_ptr(), _act_out(cache, "cache"), qa.data_ptr(), qa.stride(0),
+                                 block_table.stride(0), cache.data_ptr(), 0 if latent_t is None else latent_t.data_ptr(),
+                                 _act_out(cache, "cache"), qa.data_ptr(), qa.stride(0),
                                  rows, heads, dim, rot, rotary, rank, page_size, int(write_cache), _stream()), "latent_prep")
 
 
@@ -830,6 +838,57 @@ def shared_key_attention(q: torch.Tensor, positions: torch.Tensor, block_table: 
                                           0 if sink is None else sink.data_ptr(), out.data_ptr(), out.stride(0), heads, dk, dv,
                                           page_size, int(window), float(scale), int(heads_per_group), _stream()),
            "shared_key_attention")
+
+
+def shared_key_mfma_ok(cache_dtype: torch.dtype, dk: int, dv: int, page_size: int) -> bool:
+    """Whether the matrix-core route of the attention over shared keys takes this cache."""
+    return cache_dtype == torch.bfloat16 and dk % 8 == 0 and 0 < dv <= min(dk, 512) and page_size >= 4 and page_size % 4 == 0
+
+
+def shared_key_attention_mfma(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, tiles: Optional[torch.Tensor],
+                              num_tiles: int, cache: torch.Tensor, latent_t: torch.Tensor, sink: Optional[torch.Tensor],
+                              out: torch.Tensor, heads: int, dk: int, dv: int, page_size: int, window: int, scale: float,
+                              heads_per_group: int, nsplit: int = 1, kchunk: int = 0,
+                              partial: Optional[torch.Tensor] = None) -> None:
+    """``shared_key_attention`` on the matrix cores for a bfloat16 cache (``shared_key_mfma_ok``): queries and softmax
+    weights are rounded to bfloat16 where they enter a product, sums are 32-bit.  ``latent_t`` [pages, dv * page_size]: the
+    values transposed within their pages.  Tiles hold up to 16 / heads_per_group rows.  nsplit > 1 (tiles of one row,
+    heads_per_group 16): wave s of a tile takes keys [s * kchunk, (s+1) * kchunk) and ``partial`` (float32, at least
+    tiles * heads * nsplit * (dv + 2)) holds the pieces that a second kernel joins."""
+    _need(q, torch.float32, "q")
+    _need(out, torch.float32, "out")
+    _need(positions, torch.int32, "positions")
+    _need(block_table, torch.int32, "block_table")
+    _need(cache, torch.bfloat16, "cache")
+    _need(latent_t, torch.bfloat16, "latent_t")
+    if not shared_key_mfma_ok(cache.dtype, dk, dv, page_size):
+        raise ValueError("shared_key_attention_mfma: this cache is not for the matrix-core route")
+    if tiles is not None:
+        _need(tiles, torch.int32, "tiles")
+        if tiles.numel() < 4 * num_tiles:
+            raise ValueError("shared_key_attention_mfma: fewer tiles than said")
+    elif positions.numel() < num_tiles or block_table.shape[0] < num_tiles:
+        raise ValueError("shared_key_attention_mfma: fewer rows or block tables than implicit tiles")
+    if sink is not None:
+        _need(sink, torch.float32, "sink")
+        if sink.numel() != heads:
+            raise ValueError("shared_key_attention_mfma: a sink per head is needed")
+    if q.shape[1] != heads * dk or out.shape[1] != heads * dv:
+        raise ValueError("shared_key_attention_mfma: q or out do not fit")
+    if cache.dim() != 2 or cache.shape[1] != page_size * dk or latent_t.shape != (cache.shape[0], page_size * dv):
+        raise ValueError("shared_key_attention_mfma: cache or transposed values do not fit")
+    if nsplit > 1:
+        if partial is None:
+            raise ValueError("shared_key_attention_mfma: splits need room for their pieces")
+        _need(partial, torch.float32, "partial")
+    _check(_fn("bw_shared_key_attention_mfma")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
+                                               block_table.stride(0), 0 if tiles is None else tiles.data_ptr(), num_tiles,
+                                               cache.data_ptr(), latent_t.data_ptr(), cache.shape[0],
+                                               0 if sink is None else sink.data_ptr(), out.data_ptr(), out.stride(0), heads,
+                                               dk, dv, page_size, int(window), float(scale), int(heads_per_group), int(nsplit),
+                                               int(kchunk), 0 if partial is None else partial.data_ptr(),
+                                               0 if partial is None else partial.numel(), _stream()),
+           "shared_key_attention_mfma")
 
 
 # ------------------------------------------------------------------------------ sampling

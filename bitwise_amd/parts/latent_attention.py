@@ -21,13 +21,14 @@ from ..csrc import ops
 from .base import CacheSpec, Mixer, TensorSpec, lookup, register_mixer, POSITION_ENCODINGS
 from .linear import Linear
 
-ROWS_PER_PROMPT_TILE = 4        # 16 query vectors a workgroup: 4 rows x 4 heads, or a single token's 16 heads
+ROWS_PER_PROMPT_TILE = 4        # the 32-bit kernel: 16 query vectors a workgroup, 4 rows x 4 heads or a single token's 16 heads
+MAX_SPLITS = 32                 # pieces a single token's keys are cut into at most (each a multiple of 64 keys)
 
 
-def _tiles(ctx):
-    """(prompt tiles, count, single-token tiles, count): tiles (first row, rows, request, 0) of up to 4 consecutive rows of a
-    request; single tokens apart (their workgroups take 16 heads each).  None with a positive count: tile t is row t of
-    request t (a step of one row per request)."""
+def _tiles(ctx, rows_per_tile: int):
+    """(prompt tiles, count, single-token tiles, count): tiles (first row, rows, request, 0) of up to ``rows_per_tile``
+    consecutive rows of a request; single tokens apart (their workgroups take 16 heads each).  None with a positive
+    count: tile t is row t of request t (a step of one row per request)."""
     if getattr(ctx, "one_row_per_request", False):
         return None, 0, None, ctx.rows
 
@@ -38,13 +39,13 @@ def _tiles(ctx):
             if n == 1:
                 single.append((r0, 1, i, 0))
                 continue
-            for off in range(0, n, ROWS_PER_PROMPT_TILE):
-                many.append((r0 + off, min(ROWS_PER_PROMPT_TILE, n - off), i, 0))
+            for off in range(0, n, rows_per_tile):
+                many.append((r0 + off, min(rows_per_tile, n - off), i, 0))
         both = torch.from_numpy(np.asarray(many + single, np.int32).reshape(-1, 4)).to(ctx.device)
         return (both[:len(many)].contiguous() if many else None, len(many),
                 both[len(many):].contiguous() if single else None, len(single))
 
-    return ctx.memo(("shared_key_tiles",), make)
+    return ctx.memo(("shared_key_tiles", rows_per_tile), make)
 
 
 @register_mixer("latent_attention")
@@ -76,6 +77,14 @@ class LatentAttention(Mixer):
         self.cos = self.sin = None
         self.proj: Optional[Linear] = None
         self.o: Optional[Linear] = None
+        # bfloat16 mode: the attention runs on the matrix cores and keeps the latents a second time, transposed within
+        # their pages, as the values (the page sizes it takes: multiples of 4); the 32-bit mode reads values and keys
+        # from the one copy
+        self.on_matrix_cores = bool(runtime.bf16) and self.key_width % 8 == 0
+        # heads that share a wave's 16 query vectors in prompt portions: the power of two from the number of heads up
+        self.heads_per_group = 1
+        while self.heads_per_group < min(self.heads, 16):
+            self.heads_per_group *= 2
 
     def tensors(self) -> Dict[str, TensorSpec]:
         return {
@@ -109,7 +118,11 @@ class LatentAttention(Mixer):
         return self.proj.nbytes() + self.o.nbytes() + small + 4 * (self.rank + self.heads)
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(1, self.key_width, self.window, key_width=self.key_width, value_width=0)
+        return CacheSpec(1, self.key_width, self.window, key_width=self.key_width,
+                         value_width=self.rank if self.on_matrix_cores else 0)
+
+    def page_sizes(self):
+        return (4, 8, 16, 32, 64, 128) if self.on_matrix_cores else None
 
     def forward(self, ctx, call, h, residual) -> None:
         ws, rows = ctx.ws, ctx.rows
@@ -117,19 +130,45 @@ class LatentAttention(Mixer):
         y = ws.buffer("latent_proj", self.proj.out_features, torch.float32)
         self.proj.store(ws, h, y, rows)
         qa = ws.buffer("latent_q", self.heads * self.key_width, torch.float32)
+        mfma = self.on_matrix_cores
         ops.latent_prep(y, self.q_off, self.dkv_off, self.latent_norm, self.eps, self.cos, self.sin, ctx.positions, ctx.row_seq,
                         table, call.k_cache, qa, rows, self.heads, self.dim, self.rot, self.rotary, self.rank, ws.page_size,
-                        call.writes_cache)
+                        call.writes_cache, latent_t=call.v_cache if mfma else None)
         # the unrotated query parts into the latent's space
         ops.headwise_linear(y, self.q_off, self.dim + self.rot, self.uk_t, qa, 0, self.key_width, rows)
         lat = ws.buffer("latent_out", self.heads * self.rank, torch.float32)
-        many, n_many, single, n_single = _tiles(ctx)
-        common = (call.k_cache, self.sink, lat, self.heads, self.key_width, self.rank, ws.page_size, int(self.window or 0),
-                  self.scale)
-        if n_many:
-            ops.shared_key_attention(qa, ctx.positions, table, many, n_many, *common, 16 // ROWS_PER_PROMPT_TILE)
-        if n_single:
-            ops.shared_key_attention(qa, ctx.positions, table, single, n_single, *common, 16)
+        if mfma:
+            self._attend_on_matrix_cores(ctx, call, qa, lat, table)
+        else:
+            many, n_many, single, n_single = _tiles(ctx, ROWS_PER_PROMPT_TILE)
+            common = (call.k_cache, self.sink, lat, self.heads, self.key_width, self.rank, ws.page_size, int(self.window or 0),
+                      self.scale)
+            if n_many:
+                ops.shared_key_attention(qa, ctx.positions, table, many, n_many, *common, 16 // ROWS_PER_PROMPT_TILE)
+            if n_single:
+                ops.shared_key_attention(qa, ctx.positions, table, single, n_single, *common, 16)
         vals = ws.buffer("latent_values", self.heads * self.vdim, self.rt.act_dtype)
         ops.headwise_linear(lat, 0, self.rank, self.uv_t, vals, 0, self.vdim, rows)
         self.o.add_into(ws, vals, residual, rows)
+
+    def _attend_on_matrix_cores(self, ctx, call, qa, lat, table) -> None:
+        ws = ctx.ws
+        hg = self.heads_per_group
+        many, n_many, single, n_single = _tiles(ctx, 16 // hg)
+        common = (call.k_cache, call.v_cache, self.sink, lat, self.heads, self.key_width, self.rank, ws.page_size,
+                  int(self.window or 0), self.scale)
+        if n_many:
+            ops.shared_key_attention_mfma(qa, ctx.positions, table, many, n_many, *common, hg)
+        if n_single:
+            # Single tokens: the keys a token can have (what its block table spans) are cut into pieces of a multiple of
+            # 64, at most MAX_SPLITS of them, a wave each; few tokens with long contexts still fill the chip.  The cut
+            # depends on the table's width alone, which a captured step fixes.
+            span = table.shape[1] * ws.page_size
+            kchunk = 64 * max(1, -(-span // (64 * MAX_SPLITS)))
+            nsplit = max(1, -(-span // kchunk))
+            partial = None
+            if nsplit > 1:
+                # (room for the most pieces, for the power of two from this step's single tokens up: a few sizes at most)
+                tokens = 1 << max(0, n_single - 1).bit_length()
+                partial = ws.buffer("latent_split", tokens * MAX_SPLITS * self.heads * (self.rank + 2), torch.float32, rows=1)
+            ops.shared_key_attention_mfma(qa, ctx.positions, table, single, n_single, *common, 16, nsplit, kchunk, partial)
