@@ -99,7 +99,8 @@ int bw_linear_recurrence(int mode, const float* proj, int ldp, int q_off, int k_
                          int gate_off, int gate2_off, const float* bias, const float* bias2, float param, float qscale,
                          float* state, long long state_ld, float* out, int ldo, const int32_t* seq_rows,
                          const int32_t* slots, const int32_t* positions, int nseq, int heads, int dim, int vdim,
-                         void* stream);
+                         const int32_t* chunks, int nchunks, const int32_t* spans, int nspans, float* scan_local,
+                         float* scan_start, long long scan_floats, void* stream);
 // gate 0: sigmoid, 1: SiLU.  weight: [heads, wstride] (wstride 0: one weight vector for all heads).
 int bw_head_norm_gate(const float* o, int ldi, const float* weight, int wstride, const float* g, int ldg, int gate, void* out,
                       int out_is_bf16, int ldo, const int32_t* positions, int rows, int heads, int vdim, float eps,

@@ -80,7 +80,7 @@ _SIGS = {
                       c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_linear_recurrence": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
                              c_float, c_float, c_void_p, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                             c_int, c_int, c_int, c_void_p],
+                             c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_longlong, c_void_p],
     "bw_head_norm_gate": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int,
                           c_int, c_int, c_float, c_void_p],
     "bw_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
@@ -689,11 +689,17 @@ def norm_shift(x: torch.Tensor, weight: torch.Tensor, mix: torch.Tensor, state: 
 def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gate: torch.Tensor, gate_off: int,
                       gate2_off: int, bias: torch.Tensor, bias2: Optional[torch.Tensor], param: float, qscale: float,
                       state: torch.Tensor, out: torch.Tensor, seq_rows: torch.Tensor, slots: torch.Tensor,
-                      positions: torch.Tensor, nseq: int, heads: int, dim: int, vdim: int) -> None:
+                      positions: torch.Tensor, nseq: int, heads: int, dim: int, vdim: int, scan=None) -> None:
     """The recurrence S <- decay * S + k v^T, o = S^T (q * qscale) per head over every request's rows in order, from and
     to ``state`` [slots, elements].  RECUR_DECAY_PER_CHANNEL: decay = exp(logsigmoid(gate + bias) * param) per key
     channel (``gate`` [rows, >= gate_off + heads*dim]).  RECUR_SCALAR_GATES: capped input and forget gates per head
-    (columns gate_off + h and gate2_off + h of ``gate``), a normaliser and a running maximum in the state; param = cap."""
+    (columns gate_off + h and gate2_off + h of ``gate``), a normaliser and a running maximum in the state; param = cap.
+
+    ``scan`` = (chunks [n, 4] int32 = (first row, rows, request, 1 if the request's last chunk), n, spans [k, 3] int32 =
+    (request, its first chunk, its chunks), k, local, start): long portions run in three passes over their chunks (each
+    chunk from zero, a walk over a request's chunks that gives each its starting state, each chunk from there), with
+    ``local`` and ``start`` float32 of n * heads * (dim*vdim + dim + 2) elements each; ``seq_rows`` then carries no rows
+    for those requests (nseq may be 0).  The result differs from the one-pass order by the rounding of the walk's sums."""
     _need(proj, torch.float32, "proj")
     _need(gate, torch.float32, "gate")
     _need(bias, torch.float32, "bias")
@@ -720,11 +726,25 @@ def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_o
         raise ValueError("linear_recurrence: projections or out do not fit")
     if seq_rows.numel() < 2 * nseq or slots.numel() < nseq:
         raise ValueError("linear_recurrence: fewer request records than requests")
+    chunks = spans = local = start = None
+    nchunks = nspans = 0
+    if scan is not None:
+        chunks, nchunks, spans, nspans, local, start = scan
+        _need(chunks, torch.int32, "chunks")
+        _need(spans, torch.int32, "spans")
+        _need(local, torch.float32, "scan records")
+        _need(start, torch.float32, "scan records")
+        if chunks.numel() < 4 * nchunks or spans.numel() < 3 * nspans or start.numel() < local.numel():
+            raise ValueError("linear_recurrence: the scan's tables or records do not fit")
     _check(_fn("bw_linear_recurrence")(int(mode), proj.data_ptr(), proj.stride(0), q_off, k_off, v_off, gate.data_ptr(),
                                        gate.stride(0), gate_off, gate2_off, bias.data_ptr(),
                                        0 if bias2 is None else bias2.data_ptr(), float(param), float(qscale), state.data_ptr(),
                                        state.stride(0), out.data_ptr(), out.stride(0), seq_rows.data_ptr(), slots.data_ptr(),
-                                       positions.data_ptr(), nseq, heads, dim, vdim, _stream()), "linear_recurrence")
+                                       positions.data_ptr(), nseq, heads, dim, vdim,
+                                       0 if chunks is None else chunks.data_ptr(), nchunks,
+                                       0 if spans is None else spans.data_ptr(), nspans,
+                                       0 if local is None else local.data_ptr(), 0 if start is None else start.data_ptr(),
+                                       0 if local is None else local.numel(), _stream()), "linear_recurrence")
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, per_head_weight: bool, g: torch.Tensor, g_off: int, gate: int,

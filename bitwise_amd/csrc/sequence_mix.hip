@@ -104,6 +104,12 @@ struct RecurArgs {
   const int32_t* slots;
   const int32_t* positions;
   int heads, dim, vdim;
+  // long prompt portions in three passes (PHASE 1 to 3): chunks [n][4] = (first row, rows, request of the step, 1 if it is
+  // the request's last chunk); records of heads x (dim*vdim + dim + 2) floats per chunk: S, a vector, two scalars
+  const int32_t* chunks;
+  float* local;            // per chunk, from zero state: S, and the decay over the chunk (per channel: the product of the
+                           // decays; scalar gates: n, the maximum from -inf, the sum of the log forget gates)
+  float* start;            // per chunk: the state it starts from (S; scalar gates: n, m)
 };
 
 // One wave per (request, head, block of 64 value columns).  Lane j keeps column j of the head's state matrix in
@@ -115,39 +121,71 @@ struct RecurArgs {
 //   S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k alone, o[j] = (S^T q)[j] / (max(|n.q|, e^-m') + 1e-6).
 //   n is spread over the lanes (lane l holds n[l], n[l+64], ...); every wave of a head computes it, the wave of
 //   column block 0 stores it.
+//
+// A request's long portion can also run in three passes over chunks of its rows, which gives every chunk waves of its
+// own: PHASE 1 runs every chunk from a zero state (no read-out) and leaves the chunk's own contribution and its decay;
+// recurrence_scan_kernel walks a request's chunks in order and leaves the state each one starts from; PHASE 3 runs every
+// chunk from there with the read-out, and the request's last chunk leaves the state in the slot.  PHASE 0 is the whole
+// portion by one wave.  The passes differ from PHASE 0 by the rounding of the scan's sums only.
 #define RC 16
-template <int MODE, int DPAD>
+template <int MODE, int DPAD, int PHASE>
 __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
   constexpr bool GATES = MODE == RECUR_SCALAR_GATES;
   constexpr int NN = (DPAD + 63) / 64;
+  constexpr bool READ_OUT = PHASE != 1;
   __shared__ float qs[RC][DPAD];
   __shared__ float ks[RC][DPAD];
   __shared__ float as[GATES ? 1 : RC][GATES ? 1 : DPAD];
   __shared__ float gi[RC], gf[RC];
   __shared__ float vs[RC][64];
   const int lane = threadIdx.x;
-  const int cb = blockIdx.x, h = blockIdx.y, s = blockIdx.z;
-  const int first = a.seq_rows[2 * s], count = a.seq_rows[2 * s + 1];
-  const int slot = a.slots[s];
+  const int cb = blockIdx.x, h = blockIdx.y;
+  const int dim = a.dim, vdim = a.vdim;
+  const size_t rec = (size_t)dim * vdim + dim + 2;
+  int first, count, slot;
+  bool leaves_state = true;
+  if constexpr (PHASE == 0) {
+    const int s = blockIdx.z;
+    first = a.seq_rows[2 * s];
+    count = a.seq_rows[2 * s + 1];
+    slot = a.slots[s];
+  } else {
+    const int c = blockIdx.z;
+    first = a.chunks[4 * c];
+    count = a.chunks[4 * c + 1];
+    slot = a.slots[a.chunks[4 * c + 2]];
+    leaves_state = a.chunks[4 * c + 3] != 0;
+  }
   if (count <= 0 || slot < 0) return;
   if (a.positions[first] < 0) return;
-  const int dim = a.dim, vdim = a.vdim;
   const int j = cb * 64 + lane;
   const bool live = j < vdim;
   float* st = a.state + (size_t)slot * a.state_ld;
   float* S = st + (size_t)h * dim * vdim;
   float* nv = st + (size_t)a.heads * dim * vdim + (size_t)h * dim;
   float* mv = st + (size_t)a.heads * dim * vdim + (size_t)a.heads * dim + h;
+  // where this wave's state comes from: the slot, nothing, or the chunk's start record
+  const float* S_in = S;
+  const float* nv_in = nv;
+  const float* mv_in = mv;
+  if constexpr (PHASE == 3) {
+    S_in = a.start + ((size_t)blockIdx.z * a.heads + h) * rec;
+    nv_in = S_in + (size_t)dim * vdim;
+    mv_in = nv_in + dim;
+  }
 
   float Sreg[DPAD];
 #pragma unroll
-  for (int d = 0; d < DPAD; ++d) Sreg[d] = (live && d < dim) ? S[(size_t)d * vdim + j] : 0.0f;
-  float nreg[NN];
-  float m = 0.0f;
+  for (int d = 0; d < DPAD; ++d) Sreg[d] = (PHASE != 1 && live && d < dim) ? S_in[(size_t)d * vdim + j] : 0.0f;
+  float nreg[NN];          // scalar gates: the normaliser; per channel in PHASE 1: the product of the chunk's decays
+  float m = 0.0f, fsum = 0.0f;
   if constexpr (GATES) {
 #pragma unroll
-    for (int i = 0; i < NN; ++i) nreg[i] = (lane + 64 * i < dim) ? nv[lane + 64 * i] : 0.0f;
-    m = *mv;
+    for (int i = 0; i < NN; ++i) nreg[i] = (PHASE != 1 && lane + 64 * i < dim) ? nv_in[lane + 64 * i] : 0.0f;
+    m = PHASE == 1 ? -INFINITY : *mv_in;
+  } else {
+#pragma unroll
+    for (int i = 0; i < NN; ++i) nreg[i] = 1.0f;
   }
 
   for (int t0 = 0; t0 < count; t0 += RC) {
@@ -189,7 +227,12 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
 #pragma unroll
         for (int d = 0; d < DPAD; ++d) {
           Sreg[d] = fmaf(as[t][d], Sreg[d], ks[t][d] * v);
-          o = fmaf(Sreg[d], qs[t][d], o);
+          if constexpr (READ_OUT) o = fmaf(Sreg[d], qs[t][d], o);
+        }
+        if constexpr (PHASE == 1) {
+#pragma unroll
+          for (int i = 0; i < NN; ++i)
+            if (lane + 64 * i < DPAD) nreg[i] *= as[t][lane + 64 * i];
         }
       } else {
         const float ig = gi[t], fg = gf[t];
@@ -197,11 +240,12 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
         const float fa = bw_expf(fg + m - mn);
         const float ib = bw_expf(ig - mn);
         m = mn;
+        fsum += fg;
         const float bv = ib * vs[t][lane];
 #pragma unroll
         for (int d = 0; d < DPAD; ++d) {
           Sreg[d] = fmaf(fa, Sreg[d], ks[t][d] * bv);
-          o = fmaf(Sreg[d], qs[t][d], o);
+          if constexpr (READ_OUT) o = fmaf(Sreg[d], qs[t][d], o);
         }
         float part = 0.0f;
 #pragma unroll
@@ -212,37 +256,106 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
             part = fmaf(nreg[i], qs[t][d], part);
           }
         }
-        const float nq = wave_sum(part);
-        o = o / (fmaxf(fabsf(nq), bw_expf(-mn)) + 1e-6f);
+        if constexpr (READ_OUT) {
+          const float nq = wave_sum(part);
+          o = o / (fmaxf(fabsf(nq), bw_expf(-mn)) + 1e-6f);
+        }
       }
-      if (live) a.out[(size_t)(first + t0 + t) * a.ldo + h * vdim + j] = o;
+      if constexpr (READ_OUT) {
+        if (live) a.out[(size_t)(first + t0 + t) * a.ldo + h * vdim + j] = o;
+      }
     }
   }
+  // where the state goes: the slot (PHASE 3: from the request's last chunk only), or the chunk's own record
+  float* S_out = S;
+  float* nv_out = nv;
+  float* mv_out = mv;
+  if constexpr (PHASE == 1) {
+    S_out = a.local + ((size_t)blockIdx.z * a.heads + h) * rec;
+    nv_out = S_out + (size_t)dim * vdim;
+    mv_out = nv_out + dim;
+  }
+  if (PHASE == 3 && !leaves_state) return;
   if (live) {
 #pragma unroll
     for (int d = 0; d < DPAD; ++d)
-      if (d < dim) S[(size_t)d * vdim + j] = Sreg[d];
+      if (d < dim) S_out[(size_t)d * vdim + j] = Sreg[d];
   }
-  if constexpr (GATES) {
-    if (cb == 0) {
+  if (cb == 0 && (GATES || PHASE == 1)) {
 #pragma unroll
-      for (int i = 0; i < NN; ++i)
-        if (lane + 64 * i < dim) nv[lane + 64 * i] = nreg[i];
-      if (lane == 0) *mv = m;
+    for (int i = 0; i < NN; ++i)
+      if (lane + 64 * i < dim) nv_out[lane + 64 * i] = nreg[i];
+    if (GATES && lane == 0) {
+      mv_out[0] = m;
+      if (PHASE == 1) mv_out[1] = fsum;
     }
   }
 }
 
+// A request's chunks in order: the state each one starts from, out of the slot's state and the chunks' own contributions
+// and decays.  A thread per element of a head's record; every thread of a head walks the same scalars.
+//   per channel:   S' = decay[d] * S + S_local
+//   scalar gates:  m' = max(F + m, b), S' = e^(F + m - m') S + e^(b - m') S_local, n likewise (F: the chunk's sum of log
+//                  forget gates, b: its maximum from -inf)
 template <int MODE>
-int launch_recurrence(const RecurArgs& a, int nseq, hipStream_t s) {
-  const dim3 grid((a.vdim + 63) / 64, a.heads, nseq), block(64);
-  if (a.dim <= 16) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 16>), grid, block, 0, s, a);
-  else if (a.dim <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 32>), grid, block, 0, s, a);
-  else if (a.dim <= 64) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 64>), grid, block, 0, s, a);
-  else if (a.dim <= 128) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 128>), grid, block, 0, s, a);
-  else if (a.dim <= 256) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 256>), grid, block, 0, s, a);
+__global__ __launch_bounds__(256) void recurrence_scan_kernel(RecurArgs a, const int32_t* __restrict__ spans) {
+  constexpr bool GATES = MODE == RECUR_SCALAR_GATES;
+  const int dim = a.dim, vdim = a.vdim, h = blockIdx.y;
+  const int seq = spans[3 * blockIdx.z], c0 = spans[3 * blockIdx.z + 1], nc = spans[3 * blockIdx.z + 2];
+  const int slot = a.slots[seq];
+  if (slot < 0 || nc <= 0) return;
+  const size_t rec = (size_t)dim * vdim + dim + 2;
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  const int sd = dim * vdim;
+  const int mine = GATES ? sd + dim + 1 : sd;          // elements a head has to carry: S, and with scalar gates n and m
+  if (e >= mine) return;
+  const float* st = a.state + (size_t)slot * a.state_ld;
+  float val, m = 0.0f;
+  if (e < sd) val = st[(size_t)h * sd + e];
+  else if (e < sd + dim) val = st[(size_t)a.heads * sd + (size_t)h * dim + (e - sd)];
+  else val = 0.0f;
+  if constexpr (GATES) m = st[(size_t)a.heads * sd + (size_t)a.heads * dim + h];
+  for (int c = c0; c < c0 + nc; ++c) {
+    const float* loc = a.local + ((size_t)c * a.heads + h) * rec;
+    float* out = a.start + ((size_t)c * a.heads + h) * rec;
+    if constexpr (GATES) {
+      out[e] = e == sd + dim ? m : val;
+      const float b = loc[sd + dim], F = loc[sd + dim + 1];
+      const float mn = fmaxf(F + m, b);
+      const float ca = bw_expf(F + m - mn), cl = bw_expf(b - mn);
+      if (e < sd + dim) val = fmaf(ca, val, cl * loc[e]);
+      m = mn;
+    } else {
+      out[e] = val;
+      val = fmaf(loc[sd + e / vdim], val, loc[e]);
+    }
+  }
+}
+
+template <int MODE, int PHASE>
+int launch_recurrence(const RecurArgs& a, int units, hipStream_t s) {
+  const dim3 grid((a.vdim + 63) / 64, a.heads, units), block(64);
+  if (a.dim <= 16) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 16, PHASE>), grid, block, 0, s, a);
+  else if (a.dim <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 32, PHASE>), grid, block, 0, s, a);
+  else if (a.dim <= 64) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 64, PHASE>), grid, block, 0, s, a);
+  else if (a.dim <= 128) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 128, PHASE>), grid, block, 0, s, a);
+  else if (a.dim <= 256) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 256, PHASE>), grid, block, 0, s, a);
   else return -4;
   return BW_LAUNCH_CHECK();
+}
+
+template <int MODE>
+int launch_recurrence_passes(const RecurArgs& a, int nseq, int nchunks, const int32_t* spans, int nspans, hipStream_t s) {
+  int rc = 0;
+  if (nseq > 0) rc = launch_recurrence<MODE, 0>(a, nseq, s);
+  if (rc != 0 || nchunks <= 0) return rc;
+  rc = launch_recurrence<MODE, 1>(a, nchunks, s);
+  if (rc != 0) return rc;
+  const int mine = a.dim * a.vdim + (MODE == RECUR_SCALAR_GATES ? a.dim + 1 : 0);
+  hipLaunchKernelGGL(recurrence_scan_kernel<MODE>, dim3((mine + 255) / 256, a.heads, nspans), dim3(256), 0, s, a, spans);
+  rc = BW_LAUNCH_CHECK();
+  if (rc != 0) return rc;
+  return launch_recurrence<MODE, 3>(a, nchunks, s);
 }
 
 // ------------------------------------------------------------------------- per-head RMS norm and output gate
@@ -317,16 +430,21 @@ extern "C" int bw_linear_recurrence(int mode, const float* proj, int ldp, int q_
                                     int ldg, int gate_off, int gate2_off, const float* bias, const float* bias2, float param,
                                     float qscale, float* state, long long state_ld, float* out, int ldo,
                                     const int32_t* seq_rows, const int32_t* slots, const int32_t* positions, int nseq,
-                                    int heads, int dim, int vdim, void* stream) {
-  if (nseq <= 0) return 0;
+                                    int heads, int dim, int vdim, const int32_t* chunks, int nchunks, const int32_t* spans,
+                                    int nspans, float* scan_local, float* scan_start, long long scan_floats, void* stream) {
+  if (nseq <= 0 && nchunks <= 0) return 0;
+  if (nchunks > 0) {
+    if (chunks == nullptr || spans == nullptr || nspans <= 0 || scan_local == nullptr || scan_start == nullptr) return -2;
+    if (scan_floats < (long long)nchunks * heads * ((long long)dim * vdim + dim + 2)) return -6;
+  }
   if (heads <= 0 || dim <= 0 || vdim <= 0 || ldo < heads * vdim) return -2;
   const long long need = (long long)heads * dim * vdim + (mode == RECUR_SCALAR_GATES ? (long long)heads * dim + heads : 0);
   if (state_ld < need) return -2;
   RecurArgs a{proj, ldp, q_off, k_off, v_off, gate, ldg, gate_off, gate2_off, bias, bias2, param, qscale, state, state_ld,
-              out, ldo, seq_rows, slots, positions, heads, dim, vdim};
+              out, ldo, seq_rows, slots, positions, heads, dim, vdim, chunks, scan_local, scan_start};
   hipStream_t s = (hipStream_t)stream;
-  if (mode == RECUR_SCALAR_GATES) return launch_recurrence<RECUR_SCALAR_GATES>(a, nseq, s);
-  if (mode == RECUR_DECAY_PER_CHANNEL) return launch_recurrence<RECUR_DECAY_PER_CHANNEL>(a, nseq, s);
+  if (mode == RECUR_SCALAR_GATES) return launch_recurrence_passes<RECUR_SCALAR_GATES>(a, nseq, nchunks, spans, nspans, s);
+  if (mode == RECUR_DECAY_PER_CHANNEL) return launch_recurrence_passes<RECUR_DECAY_PER_CHANNEL>(a, nseq, nchunks, spans, nspans, s);
   return -2;
 }
 

@@ -18,11 +18,45 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional, Tuple
 
+import numpy as np
 import torch
 
 from ..csrc import ops
 from .base import Mixer, StateSpec, TensorSpec, register_mixer
 from .linear import Linear
+
+
+SCAN_CHUNK = 64          # rows of a chunk of a long portion
+SCAN_MIN_ROWS = 128      # portions from this many rows on run in three passes over chunks (shorter ones: one wave each)
+
+
+def _scan_plan(ctx):
+    """Which requests of the step bring long portions, cut into chunks: (seq_rows for the others, their count, chunks,
+    number of chunks, spans, number of spans), or None if every portion is short (a step of single tokens always is).  One
+    plan a step, shared by its layers."""
+    if getattr(ctx, "one_row_per_request", False):
+        return None
+
+    def make():
+        long = [i for i, s in enumerate(ctx.segments) if len(s.tokens) >= SCAN_MIN_ROWS]
+        if not long:
+            return None
+        short_rows = np.asarray([(ctx.seq_start[i], 0 if i in long else len(s.tokens)) for i, s in enumerate(ctx.segments)],
+                                np.int32).reshape(-1)
+        chunks, spans = [], []
+        for i in long:
+            n, r0 = len(ctx.segments[i].tokens), ctx.seq_start[i]
+            first_chunk = len(chunks)
+            for off in range(0, n, SCAN_CHUNK):
+                chunks.append((r0 + off, min(SCAN_CHUNK, n - off), i, 1 if off + SCAN_CHUNK >= n else 0))
+            spans.append((i, first_chunk, len(chunks) - first_chunk))
+        flat = np.concatenate([short_rows, np.asarray(chunks, np.int32).reshape(-1), np.asarray(spans, np.int32).reshape(-1)])
+        dev = torch.from_numpy(flat).to(ctx.device)
+        a, b = short_rows.size, short_rows.size + 4 * len(chunks)
+        any_short = len(long) < len(ctx.segments)
+        return dev[:a], (ctx.nseq if any_short else 0), dev[a:b], len(chunks), dev[b:], len(spans)
+
+    return ctx.memo(("recurrence_scan_plan",), make)
 
 
 class _MatrixMemoryMixer(Mixer):
@@ -88,6 +122,20 @@ class _MatrixMemoryMixer(Mixer):
         self.proj.store(ctx.ws, h, y, ctx.rows)
         return y
 
+    def _recur(self, ctx, call, y, gate, gate_off, gate2_off, bias, bias2, param, raw) -> None:
+        plan = _scan_plan(ctx)
+        seq_rows, nseq, scan = ctx.seq_rows, ctx.nseq, None
+        if plan is not None:
+            seq_rows, nseq, chunks, nchunks, spans, nspans = plan
+            rec = self.heads * (self.dim * self.vdim + self.dim + 2)
+            most = ctx.ws.max_rows // SCAN_CHUNK + ctx.ws.max_rows // SCAN_MIN_ROWS + 1     # chunks a step can bring
+            local = ctx.ws.buffer("recur_scan_local", most * rec, torch.float32, rows=1)
+            start = ctx.ws.buffer("recur_scan_start", most * rec, torch.float32, rows=1)
+            scan = (chunks, nchunks, spans, nspans, local, start)
+        ops.linear_recurrence(self.mode, y, self.offsets["q"], self.offsets["k"], self.offsets["v"], gate, gate_off, gate2_off,
+                              bias, bias2, param, self.qscale, call.state, raw, seq_rows, ctx.slots, ctx.positions, nseq,
+                              self.heads, self.dim, self.vdim, scan=scan)
+
     def _finish(self, ctx, y, raw, residual) -> None:
         act = ctx.ws.buffer("recur_gated", self.heads * self.vdim, self.rt.act_dtype)
         ops.head_norm_gate(raw, self.norm_weight, self.per_head_norm_weight, y, self.offsets["g"], self.gate_kind, act,
@@ -139,9 +187,7 @@ class GatedLinearAttention(_MatrixMemoryMixer):
         z = ws.buffer("gla_decay_logits", self.heads * self.dim, torch.float32)
         self.a2.store(ws, low, z, rows)
         raw = ws.buffer("recur_out", self.heads * self.vdim, torch.float32)
-        ops.linear_recurrence(self.mode, y, self.offsets["q"], self.offsets["k"], self.offsets["v"], z, 0, 0, self.a2_bias,
-                              None, 1.0 / self.tau, self.qscale, call.state, raw, ctx.seq_rows, ctx.slots, ctx.positions,
-                              ctx.nseq, self.heads, self.dim, self.vdim)
+        self._recur(ctx, call, y, z, 0, 0, self.a2_bias, None, 1.0 / self.tau, raw)
         self._finish(ctx, y, raw, residual)
 
 
@@ -183,7 +229,5 @@ class MatrixLSTM(_MatrixMemoryMixer):
     def forward(self, ctx, call, h, residual) -> None:
         y = self._project(ctx, h)
         raw = ctx.ws.buffer("recur_out", self.heads * self.vdim, torch.float32)
-        ops.linear_recurrence(self.mode, y, self.offsets["q"], self.offsets["k"], self.offsets["v"], y, self.offsets["i"],
-                              self.offsets["f"], self.i_bias, self.f_bias, self.cap, self.qscale, call.state, raw,
-                              ctx.seq_rows, ctx.slots, ctx.positions, ctx.nseq, self.heads, self.dim, self.vdim)
+        self._recur(ctx, call, y, y, self.offsets["i"], self.offsets["f"], self.i_bias, self.f_bias, self.cap, raw)
         self._finish(ctx, y, raw, residual)

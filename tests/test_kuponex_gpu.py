@@ -183,6 +183,28 @@ def test_long_decoding(folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_portions_beside_short_ones(folders, dtype):
+    """Portions long enough for the recurrences' three passes over chunks (whole, cut at and beside a chunk's edge), alone and
+    in one step with a short portion and a single token of other requests."""
+    name = "wide"
+    toks = tokens_for(name, 330, 31)
+    want = plain(name, folders[name], toks, dtype)
+    rp = replayer(folders[name], dtype, 1024)
+    for k, cuts in enumerate(([330], [129, 201], [128, 128, 74], [191, 130])):
+        assert close(run_cut(rp, f"w{k}", toks, cuts), want, dtype), cuts
+    small, one = tokens_for(name, 9, 32), tokens_for(name, 3, 33)
+    rp.step([{"id": "one", "tokens": one[:2], "want": []}])
+    lg = rp.step([{"id": "small", "tokens": small[:5], "want": [4]}, {"id": "long", "tokens": toks[:260], "want": [0, 127, 128, 259]},
+                  {"id": "one", "tokens": one[2:], "want": [0]}])
+    assert close(lg[1:5], want[[0, 127, 128, 259]], dtype)
+    assert close(lg[:1], plain(name, folders[name], small, dtype)[4:5], dtype)
+    assert close(lg[5:], plain(name, folders[name], one, dtype)[2:], dtype)
+    lg = rp.step([{"id": "long", "tokens": toks[260:], "want": [0, 69]}, {"id": "small", "tokens": small[5:], "want": [3]}], ["long", "small", "one"])
+    assert close(lg[:2], want[[260, 329]], dtype) and close(lg[2:], plain(name, folders[name], small, dtype)[8:], dtype)
+    assert rp.manager.all_free()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_through_the_engine(folders, dtype):
     """bw.generate with the engine's scheduler, a small token budget and a small page pool: the tokens of the plain
     implementation, which recomputes the whole sequence for every token."""
