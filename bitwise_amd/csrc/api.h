@@ -110,7 +110,7 @@ int bw_glu(const float* gate_up, void* h, int out_is_bf16, int rows, int inter, 
 // Attention over a compressed cache shared by all heads (latent_attention.hip).
 int bw_latent_prep(const float* proj, int ldp, int q_off, int dkv_off, const float* norm_w, float eps,
                    const float* cos_table, const float* sin_table, const int32_t* positions, const int32_t* row_seq,
-                   const int32_t* block_table, int table_stride, void* cache, void* latent_t, int cache_is_bf16, float* qa, int ldqa,
+                   const int32_t* block_table, int table_stride, void* cache, void* latent_t, int cache_is_bf16, void* qa, int qa_is_bf16, int ldqa,
                    int rows, int heads, int dim, int rot, int rotary, int rank, int page_size, int write_cache,
                    void* stream);
 int bw_headwise_linear(const float* x, int ldx, int xhs, const void* wt, int w_is_bf16, int in, int outn, void* out,
@@ -119,7 +119,7 @@ int bw_shared_key_attention(const float* q, int ldq, const int32_t* positions, c
                             int table_stride, const int32_t* tiles, int num_tiles, const void* cache, int cache_is_bf16,
                             int num_pages, const float* sink, float* out, int ldo, int heads, int dk, int dv,
                             int page_size, int window, float scale, int heads_per_group, void* stream);
-int bw_shared_key_attention_mfma(const float* q, int ldq, const int32_t* positions, const int32_t* block_table,
+int bw_shared_key_attention_mfma(const void* q, int ldq, const int32_t* positions, const int32_t* block_table,
                                  int table_stride, const int32_t* tiles, int num_tiles, const void* cache,
                                  const void* latent_t, int num_pages, const float* sink, float* out, int ldo, int heads,
                                  int dk, int dv, int page_size, int window, float scale, int heads_per_group, int nsplit,

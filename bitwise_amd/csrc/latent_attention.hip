@@ -43,8 +43,8 @@ struct PrepArgs {
   const int32_t* row_seq;
   const int32_t* block_table;
   int table_stride;
-  float* qa;             // [rows, ldqa]: head h at h * (rank + rot); the rotated part goes to its last rot elements
-  int ldqa;
+  void* qa;              // [rows, ldqa] (32-bit, or bfloat16 for the matrix-core attention): head h at h * (rank + rot); the
+  int ldqa, qa_is_bf16;  // rotated part goes to its last rot elements
   int heads, dim, rot, rotary, rank, page_size, write_cache;
 };
 
@@ -91,7 +91,9 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(PrepArgs a, CT* __rest
     if (i < half) v = qr[i] * ct[i] - qr[i + half] * st[i];
     else if (i < a.rotary) v = qr[i] * ct[i - half] + qr[i - half] * st[i - half];
     else v = qr[i];
-    a.qa[(size_t)row * a.ldqa + h * width + a.rank + i] = v;
+    const size_t at = (size_t)row * a.ldqa + h * width + a.rank + i;
+    if (a.qa_is_bf16) reinterpret_cast<bf16_t*>(a.qa)[at] = f32_to_bf16(v);
+    else reinterpret_cast<float*>(a.qa)[at] = v;
   }
 }
 
@@ -100,32 +102,51 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(PrepArgs a, CT* __rest
 // out[r][h*ohs + o] = sum_i wt[h][i][o] * x[r][h*xhs + i]: the weights lie input-major, so that neighbouring threads
 // (outputs) read neighbouring weights; HL_ROWS rows share every weight that is loaded.  One fused multiply-add chain
 // per output, i ascending.
+// A workgroup is 64 outputs by four quarters of the inner size (a wave a quarter, eight weights asked for at a time); the
+// quarters' sums meet in LDS and are added in quarter order.
 #define HL_ROWS 8
 template <typename WT, typename OT>
 __global__ __launch_bounds__(256) void headwise_linear_kernel(const float* __restrict__ x, int ldx, int xhs,
                                                               const WT* __restrict__ wt, int in, int outn,
                                                               OT* __restrict__ out, int ldo, int ohs, int rows) {
-  extern __shared__ float hl_x[];      // [HL_ROWS][in]
+  extern __shared__ float hl_x[];      // [HL_ROWS][in], then [4][HL_ROWS][64] partial sums
+  float* hl_part = hl_x + HL_ROWS * in;
   const int r0 = blockIdx.x * HL_ROWS, h = blockIdx.y;
-  const int o = blockIdx.z * 256 + threadIdx.x;
+  const int lane = threadIdx.x & 63, quarter = wave_index();
+  const int o = blockIdx.z * 64 + lane;
   for (int e = threadIdx.x; e < HL_ROWS * in; e += 256) {
     const int r = e / in, i = e % in;
     hl_x[e] = (r0 + r < rows) ? x[(size_t)(r0 + r) * ldx + h * xhs + i] : 0.0f;
   }
   __syncthreads();
-  if (o >= outn) return;
   float acc[HL_ROWS];
 #pragma unroll
   for (int r = 0; r < HL_ROWS; ++r) acc[r] = 0.0f;
-  const WT* wp = wt + (size_t)h * in * outn + o;
-  for (int i = 0; i < in; ++i) {
-    const float w = load_f(wp + (size_t)i * outn);
+  const int per = (in + 3) / 4;
+  const int i0 = quarter * per, i1 = min(in, i0 + per);
+  const WT* wp = wt + (size_t)h * in * outn + min(o, outn - 1);
+  for (int i = i0; i < i1; i += 8) {
+    float w[8];
 #pragma unroll
-    for (int r = 0; r < HL_ROWS; ++r) acc[r] = fmaf(hl_x[r * in + i], w, acc[r]);
+    for (int u = 0; u < 8; ++u) w[u] = load_f(wp + (size_t)min(i + u, i1 - 1) * outn);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (i + u < i1) {
+#pragma unroll
+        for (int r = 0; r < HL_ROWS; ++r) acc[r] = fmaf(hl_x[r * in + i + u], w[u], acc[r]);
+      }
+    }
   }
 #pragma unroll
-  for (int r = 0; r < HL_ROWS; ++r)
-    if (r0 + r < rows) store_f(out + (size_t)(r0 + r) * ldo + h * ohs + o, acc[r]);
+  for (int r = 0; r < HL_ROWS; ++r) hl_part[(quarter * HL_ROWS + r) * 64 + lane] = acc[r];
+  __syncthreads();
+  if (quarter != 0 || o >= outn) return;
+#pragma unroll
+  for (int r = 0; r < HL_ROWS; ++r) {
+    const float sum = ((hl_part[r * 64 + lane] + hl_part[(HL_ROWS + r) * 64 + lane]) + hl_part[(2 * HL_ROWS + r) * 64 + lane]) +
+                      hl_part[(3 * HL_ROWS + r) * 64 + lane];
+    if (r0 + r < rows) store_f(out + (size_t)(r0 + r) * ldo + h * ohs + o, sum);
+  }
 }
 
 // ------------------------------------------------------------------------- attention over shared keys
@@ -335,7 +356,7 @@ int launch_shared_key(const SharedKeyArgs& a, const CT* cache, int num_tiles, hi
 // query (lane mod 16).  With nsplit > 1 a wave takes kchunk keys and leaves (maximum, denominator, sums) for
 // shared_key_combine_kernel; the sink joins where the result is finished.
 struct MfmaAttnArgs {
-  const float* q;
+  const bf16_t* q;         // [rows, ldq] bfloat16: head h at h * dk
   int ldq;
   const int32_t* positions;
   const int32_t* block_table;
@@ -390,11 +411,16 @@ __global__ __launch_bounds__(64) void shared_key_attention_mfma_kernel(MfmaAttnA
   const int qpos = qok ? pos0 + rl : -1;
   const int qlo = a.window > 0 ? max(0, qpos - a.window + 1) : 0;
   const int dkp = (a.dk + 31) & ~31, qstride = dkp + 8;
-  for (int e = lane; e < 16 * dkp; e += 64) {
-    const int qn = e / dkp, d = e % dkp;
-    const int r2 = qn / a.hg, h2 = h0 + qn % a.hg;
-    const float v = (r2 < nr && h2 < a.heads && d < a.dk) ? a.q[(size_t)(r0 + r2) * a.ldq + h2 * a.dk + d] : 0.0f;
-    qs[qn * qstride + d] = f32_to_bf16(v);
+  {
+    const int groups = dkp >> 3;             // 16-byte groups of a query vector (dk is a multiple of 8)
+#pragma unroll 4
+    for (int e = lane; e < 16 * groups; e += 64) {
+      const int qn = e / groups, d = (e % groups) * 8;
+      const int r2 = qn / a.hg, h2 = h0 + qn % a.hg;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (r2 < nr && h2 < a.heads && d < a.dk) v = *reinterpret_cast<const u32x4*>(a.q + (size_t)(r0 + r2) * a.ldq + h2 * a.dk + d);
+      *reinterpret_cast<u32x4*>(qs + qn * qstride + d) = v;
+    }
   }
   __syncthreads();
 
@@ -423,13 +449,20 @@ __global__ __launch_bounds__(64) void shared_key_attention_mfma_kernel(MfmaAttnA
     f32x4 st[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) st[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    for (int d0 = 8 * g; d0 < dkp; d0 += 32) {
-      const u32x4 qf = *reinterpret_cast<const u32x4*>(qs + n * qstride + d0);
-      u32x4 kf[4];
+    for (int d1 = 8 * g; d1 < dkp; d1 += 128) {          // four steps of 32 elements: their 16 loads are in flight together
+      u32x4 kf[4][4], qf[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) kf[u] = d0 < dk ? *reinterpret_cast<const u32x4*>(krow[u] + d0) : (u32x4){0u, 0u, 0u, 0u};
+      for (int s4 = 0; s4 < 4; ++s4) {
+        const int d0 = d1 + 32 * s4;
+        qf[s4] = d0 < dkp ? *reinterpret_cast<const u32x4*>(qs + n * qstride + d0) : (u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int u = 0; u < 4; ++u) st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u]), as_bf16x8(qf), st[u], 0, 0, 0);
+        for (int u = 0; u < 4; ++u) kf[s4][u] = d0 < dk ? *reinterpret_cast<const u32x4*>(krow[u] + d0) : (u32x4){0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[s4][u]), as_bf16x8(qf[s4]), st[u], 0, 0, 0);
     }
     // this lane: query n, keys kb0 + 16u + 4g + i
     float mx = -INFINITY;
@@ -533,19 +566,26 @@ __global__ __launch_bounds__(64) void shared_key_combine_kernel(MfmaAttnArgs a) 
   const float* part = a.partial + ((size_t)t * a.heads + h) * a.nsplit * (a.dv + 2);
   const int live = min(a.nsplit, a.positions[r0] / a.kchunk + 1);      // splits beyond the row's position hold nothing
   const float sk = a.sink != nullptr ? a.sink[h] : -INFINITY;
-  float mt = sk;
-  for (int s = 0; s < live; ++s) mt = fmaxf(mt, part[(size_t)s * (a.dv + 2)]);
-  float lt = sk == -INFINITY ? 0.0f : fast_exp(sk - mt);
-  for (int s = 0; s < live; ++s) {
-    const float ms = part[(size_t)s * (a.dv + 2)];
-    if (ms != -INFINITY) lt += part[(size_t)s * (a.dv + 2) + 1] * fast_exp(ms - mt);
-  }
+  // lane s holds split s's maximum and denominator (at most 64 splits); the weights of the splits go through LDS
+  __shared__ float wgt[64];
+  const int lane = threadIdx.x;
+  const float ms = lane < live ? part[(size_t)lane * (a.dv + 2)] : -INFINITY;
+  const float ls = lane < live ? part[(size_t)lane * (a.dv + 2) + 1] : 0.0f;
+  const float mt = fmaxf(sk, wave_max(ms));
+  const float ws = ms == -INFINITY ? 0.0f : fast_exp(ms - mt);
+  const float lt = wave_sum(ls * ws) + (sk == -INFINITY ? 0.0f : fast_exp(sk - mt));
+  wgt[lane] = ws;
+  __syncthreads();
   const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
-  for (int d = threadIdx.x; d < a.dv; d += 64) {
+  for (int d = lane; d < a.dv; d += 64) {
     float o = 0.0f;
-    for (int s = 0; s < live; ++s) {
-      const float ms = part[(size_t)s * (a.dv + 2)];
-      if (ms != -INFINITY) o = fmaf(part[(size_t)s * (a.dv + 2) + 2 + d], fast_exp(ms - mt), o);
+    for (int s0 = 0; s0 < live; s0 += 8) {
+      float pv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) pv[u] = part[(size_t)min(s0 + u, live - 1) * (a.dv + 2) + 2 + d];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < live && wgt[s0 + u] != 0.0f) o = fmaf(pv[u], wgt[s0 + u], o);
     }
     a.out[(size_t)r0 * a.ldo + h * a.dv + d] = o * inv;
   }
@@ -570,13 +610,13 @@ int launch_shared_key_mfma(const MfmaAttnArgs& a, const bf16_t* kc, const bf16_t
 extern "C" int bw_latent_prep(const float* proj, int ldp, int q_off, int dkv_off, const float* norm_w, float eps,
                               const float* cos_table, const float* sin_table, const int32_t* positions,
                               const int32_t* row_seq, const int32_t* block_table, int table_stride, void* cache,
-                              void* latent_t, int cache_is_bf16, float* qa, int ldqa, int rows, int heads, int dim, int rot, int rotary,
+                              void* latent_t, int cache_is_bf16, void* qa, int qa_is_bf16, int ldqa, int rows, int heads, int dim, int rot, int rotary,
                               int rank, int page_size, int write_cache, void* stream) {
   if (rows <= 0) return 0;
   if (heads <= 0 || dim < 0 || rot < 0 || rotary < 0 || rotary > rot || (rotary & 1) || rank <= 0 || page_size <= 0) return -2;
   if (ldqa < heads * (rank + rot)) return -2;
   PrepArgs a{proj, ldp, q_off, dkv_off, norm_w, eps, cos_table, sin_table, positions, row_seq, block_table, table_stride,
-             qa, ldqa, heads, dim, rot, rotary, rank, page_size, write_cache};
+             qa, ldqa, qa_is_bf16, heads, dim, rot, rotary, rank, page_size, write_cache};
   hipStream_t s = (hipStream_t)stream;
   if (cache_is_bf16) hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, a, (bf16_t*)cache, (bf16_t*)latent_t);
   else hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(rows), dim3(256), 0, s, a, (float*)cache, (float*)latent_t);
@@ -586,10 +626,10 @@ extern "C" int bw_latent_prep(const float* proj, int ldp, int q_off, int dkv_off
 extern "C" int bw_headwise_linear(const float* x, int ldx, int xhs, const void* wt, int w_is_bf16, int in, int outn,
                                   void* out, int out_is_bf16, int ldo, int ohs, int rows, int heads, void* stream) {
   if (rows <= 0 || heads <= 0 || outn <= 0) return 0;
-  if (in <= 0 || (size_t)HL_ROWS * in * sizeof(float) > 60 * 1024) return -2;
+  if (in <= 0 || (size_t)HL_ROWS * in * sizeof(float) > 48 * 1024) return -2;
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid((rows + HL_ROWS - 1) / HL_ROWS, heads, (outn + 255) / 256), block(256);
-  const size_t bytes = (size_t)HL_ROWS * in * sizeof(float);
+  const dim3 grid((rows + HL_ROWS - 1) / HL_ROWS, heads, (outn + 63) / 64), block(256);
+  const size_t bytes = (size_t)HL_ROWS * (in + 4 * 64) * sizeof(float);
   if (w_is_bf16) {
     if (out_is_bf16)
       hipLaunchKernelGGL((headwise_linear_kernel<bf16_t, bf16_t>), grid, block, bytes, s, x, ldx, xhs, (const bf16_t*)wt, in, outn,
@@ -627,7 +667,7 @@ extern "C" int bw_shared_key_attention(const float* q, int ldq, const int32_t* p
 // The matrix-core route: bfloat16 cache with key vectors of a multiple of 8 elements, pages of a multiple of 4 slots, and the
 // transposed latents beside it.  nsplit > 1 (single-row tiles, 16 heads a group): every wave takes kchunk keys (a multiple
 // of 64) and ``partial`` holds tiles * heads * nsplit * (dv + 2) floats.
-extern "C" int bw_shared_key_attention_mfma(const float* q, int ldq, const int32_t* positions, const int32_t* block_table,
+extern "C" int bw_shared_key_attention_mfma(const void* q, int ldq, const int32_t* positions, const int32_t* block_table,
                                             int table_stride, const int32_t* tiles, int num_tiles, const void* cache,
                                             const void* latent_t, int num_pages, const float* sink, float* out, int ldo,
                                             int heads, int dk, int dv, int page_size, int window, float scale,
@@ -636,13 +676,14 @@ extern "C" int bw_shared_key_attention_mfma(const float* q, int ldq, const int32
   if (num_tiles <= 0) return 0;
   if (heads <= 0 || dk <= 0 || (dk % 8) || dv <= 0 || dv > dk || dv > 512 || page_size < 4 || (page_size % 4) || num_pages <= 0) return -2;
   if (heads_per_group < 1 || heads_per_group > 16 || (16 % heads_per_group)) return -2;
-  if (ldq < heads * dk || ldo < heads * dv || nsplit < 1) return -2;
+  if (ldq < heads * dk || (ldq % 8) || ldo < heads * dv || nsplit < 1 || nsplit > 64) return -2;
+  if (reinterpret_cast<uintptr_t>(q) & 15) return -3;
   if (nsplit > 1) {
     if (heads_per_group != 16 || kchunk < 64 || (kchunk % 64) || partial == nullptr) return -2;
     if (partial_floats < (long long)num_tiles * heads * nsplit * (dv + 2)) return -6;
   }
   if ((reinterpret_cast<uintptr_t>(cache) & 15) || (reinterpret_cast<uintptr_t>(latent_t) & 7)) return -3;
-  MfmaAttnArgs a{q, ldq, positions, block_table, table_stride, tiles, sink, out, ldo, partial, heads, dk, dv, page_size, window,
+  MfmaAttnArgs a{(const bf16_t*)q, ldq, positions, block_table, table_stride, tiles, sink, out, ldo, partial, heads, dk, dv, page_size, window,
                  heads_per_group, num_pages, nsplit, kchunk, scale};
   return launch_shared_key_mfma(a, (const bf16_t*)cache, (const bf16_t*)latent_t, num_tiles, (hipStream_t)stream);
 }

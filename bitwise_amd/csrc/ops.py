@@ -88,7 +88,7 @@ _SIGS = {
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
                                      c_void_p, c_longlong, c_void_p],
     "bw_latent_prep": [c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                       c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                       c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                        c_void_p],
     "bw_headwise_linear": [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
                            c_int, c_void_p],
@@ -787,7 +787,6 @@ def latent_prep(proj: torch.Tensor, q_off: int, dkv_off: int, norm_w: torch.Tens
     _need(norm_w, torch.float32, "norm weight")
     _need(cos, torch.float32, "cos table")
     _need(sin, torch.float32, "sin table")
-    _need(qa, torch.float32, "qa")
     for t, what in ((positions, "positions"), (row_seq, "row_seq"), (block_table, "block_table")):
         _need(t, torch.int32, what)
     width = rank + rot
@@ -805,7 +804,7 @@ def latent_prep(proj: torch.Tensor, q_off: int, dkv_off: int, norm_w: torch.Tens
     _check(_fn("bw_latent_prep")(proj.data_ptr(), proj.stride(0), q_off, dkv_off, norm_w.data_ptr(), float(eps), cos.data_ptr(),
                                  sin.data_ptr(), positions.data_ptr(), row_seq.data_ptr(), block_table.data_ptr(),
                                  block_table.stride(0), cache.data_ptr(), 0 if latent_t is None else latent_t.data_ptr(),
-                                 _act_out(cache, "cache"), qa.data_ptr(), qa.stride(0),
+                                 _act_out(cache, "cache"), qa.data_ptr(), _act_out(qa, "qa"), qa.stride(0),
                                  rows, heads, dim, rot, rotary, rank, page_size, int(write_cache), _stream()), "latent_prep")
 
 
@@ -871,11 +870,11 @@ def shared_key_attention_mfma(q: torch.Tensor, positions: torch.Tensor, block_ta
                               heads_per_group: int, nsplit: int = 1, kchunk: int = 0,
                               partial: Optional[torch.Tensor] = None) -> None:
     """``shared_key_attention`` on the matrix cores for a bfloat16 cache (``shared_key_mfma_ok``): queries and softmax
-    weights are rounded to bfloat16 where they enter a product, sums are 32-bit.  ``latent_t`` [pages, dv * page_size]: the
+    weights are rounded to bfloat16 where they enter a product (``q`` arrives as bfloat16), sums are 32-bit.  ``latent_t`` [pages, dv * page_size]: the
     values transposed within their pages.  Tiles hold up to 16 / heads_per_group rows.  nsplit > 1 (tiles of one row,
     heads_per_group 16): wave s of a tile takes keys [s * kchunk, (s+1) * kchunk) and ``partial`` (float32, at least
     tiles * heads * nsplit * (dv + 2)) holds the pieces that a second kernel joins."""
-    _need(q, torch.float32, "q")
+    _need(q, torch.bfloat16, "q")
     _need(out, torch.float32, "out")
     _need(positions, torch.int32, "positions")
     _need(block_table, torch.int32, "block_table")

@@ -59,9 +59,57 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict
   const int slot = slots[seq];
   if (slot < 0 || count <= 0) return;
   const float* xr = x + (size_t)row * ldx;
-  const float inv = 1.0f / sqrtf(row_sumsq(xr, dim, lane) / (float)dim + eps);
   float* st = state + (size_t)slot * state_ld;
   OT* o = out + (size_t)row * ldo;
+  if ((dim & 3) == 0 && (ldx & 3) == 0 && (ldo & 3) == 0 && (state_ld & 3) == 0) {
+    // rows of whole 16-byte vectors: lane l owns vectors l, l+64, ...; four of them (and of everything that goes with them) are
+    // asked for before the first is used
+    const int nvec = dim >> 2;
+    const bool is_first = row == first;
+    const int last = first + count - 1;
+    const f32x4* xv = reinterpret_cast<const f32x4*>(xr);
+    const f32x4* pv = is_first ? reinterpret_cast<const f32x4*>(st) : reinterpret_cast<const f32x4*>(xr - ldx);
+    const f32x4* lv = reinterpret_cast<const f32x4*>(x + (size_t)last * ldx);
+    const f32x4* wv = reinterpret_cast<const f32x4*>(w);
+    const f32x4* mv = reinterpret_cast<const f32x4*>(mix);
+    const float inv = 1.0f / sqrtf(row_sumsq_vec(xv, nvec, lane) / (float)dim + eps);
+    const float invp = is_first ? 1.0f : 1.0f / sqrtf(row_sumsq_vec(pv, nvec, lane) / (float)dim + eps);
+    const float invl = !is_first || last == row ? inv : 1.0f / sqrtf(row_sumsq_vec(lv, nvec, lane) / (float)dim + eps);
+    constexpr int UN = 4;
+    for (int c0 = 0; c0 < nvec; c0 += 64 * UN) {
+      f32x4 xq[UN], pq[UN], lq[UN], wq[UN], mq[UN];
+#pragma unroll
+      for (int jj = 0; jj < UN; ++jj) {
+        const int c = min(c0 + 64 * jj + lane, nvec - 1);
+        xq[jj] = xv[c];
+        pq[jj] = pv[c];
+        wq[jj] = wv[c];
+        mq[jj] = mv[c];
+        lq[jj] = is_first ? lv[c] : xq[jj];
+      }
+#pragma unroll
+      for (int jj = 0; jj < UN; ++jj) {
+        const int c = c0 + 64 * jj + lane;
+        if (c >= nvec) continue;
+        f32x4 r, keep;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float h = (xq[jj][e] * inv) * wq[jj][e];
+          const float hp = is_first ? pq[jj][e] : (pq[jj][e] * invp) * wq[jj][e];
+          r[e] = fmaf(hp - h, mq[jj][e], h);
+          keep[e] = (lq[jj][e] * invl) * wq[jj][e];
+        }
+        if constexpr (sizeof(OT) == 2) {
+          *reinterpret_cast<u32x2*>(o + 4 * c) = (u32x2){pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+        } else {
+          *reinterpret_cast<f32x4*>(o + 4 * c) = r;
+        }
+        if (is_first) reinterpret_cast<f32x4*>(st)[c] = keep;
+      }
+    }
+    return;
+  }
+  const float inv = 1.0f / sqrtf(row_sumsq(xr, dim, lane) / (float)dim + eps);
   if (row != first) {
     const float* xp = xr - ldx;
     const float invp = 1.0f / sqrtf(row_sumsq(xp, dim, lane) / (float)dim + eps);

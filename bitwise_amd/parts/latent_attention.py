@@ -129,8 +129,9 @@ class LatentAttention(Mixer):
         table = ctx.block_tables[call.group]
         y = ws.buffer("latent_proj", self.proj.out_features, torch.float32)
         self.proj.store(ws, h, y, rows)
-        qa = ws.buffer("latent_q", self.heads * self.key_width, torch.float32)
         mfma = self.on_matrix_cores
+        # (the matrix-core kernel takes its queries rounded to bfloat16, so they are stored that way at once)
+        qa = ws.buffer("latent_q", self.heads * self.key_width, torch.bfloat16 if mfma else torch.float32)
         ops.latent_prep(y, self.q_off, self.dkv_off, self.latent_norm, self.eps, self.cos, self.sin, ctx.positions, ctx.row_seq,
                         table, call.k_cache, qa, rows, self.heads, self.dim, self.rot, self.rotary, self.rank, ws.page_size,
                         call.writes_cache, latent_t=call.v_cache if mfma else None)
