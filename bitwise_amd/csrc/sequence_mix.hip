@@ -160,7 +160,7 @@ struct RecurArgs {
   float* start;            // per chunk: the state it starts from (S; scalar gates: n, m)
 };
 
-// One wave per (request, head, block of 64 value columns).  Lane j keeps column j of the head's state matrix in
+// One wave per (request, head, block of 64 value columns; 32 for heads of more than 64 key channels).  Lane j keeps column j of the head's state matrix in
 // registers (one element per key channel), so the read-out S^T q needs no exchange between lanes; the tokens' q, k and
 // decays come through LDS in chunks of RC tokens and are read from there by all lanes at once.
 //
@@ -181,6 +181,10 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
   constexpr bool GATES = MODE == RECUR_SCALAR_GATES;
   constexpr int NN = (DPAD + 63) / 64;
   constexpr bool READ_OUT = PHASE != 1;
+  // heads of 128 key channels and more: a column's channels are split over two lanes (lane l and l + 32 hold the two halves
+  // of column l mod 32), so that a lane's part of the state fits its registers; the halves' read-outs are added lower + upper
+  constexpr int SPLIT = DPAD >= 128 ? 2 : 1;
+  constexpr int DH = DPAD / SPLIT, COLS = 64 / SPLIT;
   __shared__ float qs[RC][DPAD];
   __shared__ float ks[RC][DPAD];
   __shared__ float as[GATES ? 1 : RC][GATES ? 1 : DPAD];
@@ -206,7 +210,8 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
   }
   if (count <= 0 || slot < 0) return;
   if (a.positions[first] < 0) return;
-  const int j = cb * 64 + lane;
+  const int col = lane % COLS, dbase = (lane / COLS) * DH;
+  const int j = cb * COLS + col;
   const bool live = j < vdim;
   float* st = a.state + (size_t)slot * a.state_ld;
   float* S = st + (size_t)h * dim * vdim;
@@ -222,9 +227,9 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
     mv_in = nv_in + dim;
   }
 
-  float Sreg[DPAD];
+  float Sreg[DH];
 #pragma unroll
-  for (int d = 0; d < DPAD; ++d) Sreg[d] = (PHASE != 1 && live && d < dim) ? S_in[(size_t)d * vdim + j] : 0.0f;
+  for (int d = 0; d < DH; ++d) Sreg[d] = (PHASE != 1 && live && dbase + d < dim) ? S_in[(size_t)(dbase + d) * vdim + j] : 0.0f;
   float nreg[NN];          // scalar gates: the normaliser; per channel in PHASE 1: the product of the chunk's decays
   float m = 0.0f, fsum = 0.0f;
   if constexpr (GATES) {
@@ -239,20 +244,28 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
   for (int t0 = 0; t0 < count; t0 += RC) {
     const int tc = min(RC, count - t0);
     __syncthreads();
-    for (int e = lane; e < tc * DPAD; e += 64) {
-      const int t = e / DPAD, d = e % DPAD;
-      const size_t row = (size_t)(first + t0 + t);
-      const float* pr = a.proj + row * a.ldp;
-      const bool in = d < dim;
-      qs[t][d] = in ? pr[a.q_off + h * dim + d] * a.qscale : 0.0f;
-      ks[t][d] = in ? pr[a.k_off + h * dim + d] : 0.0f;
-      if constexpr (!GATES) {
-        float al = 0.0f;
-        if (in) {
-          const float z = a.gate[row * a.ldg + a.gate_off + h * dim + d] + a.bias[h * dim + d];
-          al = bw_expf(log_sigmoid(z) * a.param);
-        }
-        as[t][d] = al;
+    // eight elements a lane at a time: their loads are all asked for before the first is used
+    for (int e0 = 0; e0 < tc * DPAD; e0 += 64 * 8) {
+      float qv[8], kv[8], zv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int e = e0 + 64 * u + lane;
+        const int t = e / DPAD, d = e % DPAD;
+        const bool in = e < tc * DPAD && d < dim;
+        const size_t row = (size_t)(first + t0 + min(t, tc - 1));
+        const float* pr = a.proj + row * a.ldp;
+        qv[u] = in ? pr[a.q_off + h * dim + d] : 0.0f;
+        kv[u] = in ? pr[a.k_off + h * dim + d] : 0.0f;
+        if constexpr (!GATES) zv[u] = in ? a.gate[row * a.ldg + a.gate_off + h * dim + d] + a.bias[h * dim + d] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int e = e0 + 64 * u + lane;
+        if (e >= tc * DPAD) continue;
+        const int t = e / DPAD, d = e % DPAD;
+        qs[t][d] = qv[u] * a.qscale;
+        ks[t][d] = kv[u];
+        if constexpr (!GATES) as[t][d] = d < dim ? bw_expf(log_sigmoid(zv[u]) * a.param) : 0.0f;
       }
     }
     if constexpr (GATES) {
@@ -263,19 +276,21 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
         gf[lane] = log_sigmoid(cap * tanhf((pr[a.gate2_off + h] + a.bias2[h]) / cap));
       }
     }
-    // (each lane writes and reads its own column of vs)
+    // (a column's lanes read what its first lane wrote)
+    if (lane < COLS) {
 #pragma unroll
-    for (int t = 0; t < RC; ++t)
-      vs[t][lane] = (live && t < tc) ? a.proj[(size_t)(first + t0 + t) * a.ldp + a.v_off + h * vdim + j] : 0.0f;
+      for (int t = 0; t < RC; ++t)
+        vs[t][col] = (live && t < tc) ? a.proj[(size_t)(first + t0 + t) * a.ldp + a.v_off + h * vdim + j] : 0.0f;
+    }
     __syncthreads();
     for (int t = 0; t < tc; ++t) {
       float o = 0.0f;
       if constexpr (!GATES) {
-        const float v = vs[t][lane];
+        const float v = vs[t][col];
 #pragma unroll
-        for (int d = 0; d < DPAD; ++d) {
-          Sreg[d] = fmaf(as[t][d], Sreg[d], ks[t][d] * v);
-          if constexpr (READ_OUT) o = fmaf(Sreg[d], qs[t][d], o);
+        for (int d = 0; d < DH; ++d) {
+          Sreg[d] = fmaf(as[t][dbase + d], Sreg[d], ks[t][dbase + d] * v);
+          if constexpr (READ_OUT) o = fmaf(Sreg[d], qs[t][dbase + d], o);
         }
         if constexpr (PHASE == 1) {
 #pragma unroll
@@ -289,11 +304,11 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
         const float ib = bw_expf(ig - mn);
         m = mn;
         fsum += fg;
-        const float bv = ib * vs[t][lane];
+        const float bv = ib * vs[t][col];
 #pragma unroll
-        for (int d = 0; d < DPAD; ++d) {
-          Sreg[d] = fmaf(fa, Sreg[d], ks[t][d] * bv);
-          if constexpr (READ_OUT) o = fmaf(Sreg[d], qs[t][d], o);
+        for (int d = 0; d < DH; ++d) {
+          Sreg[d] = fmaf(fa, Sreg[d], ks[t][dbase + d] * bv);
+          if constexpr (READ_OUT) o = fmaf(Sreg[d], qs[t][dbase + d], o);
         }
         float part = 0.0f;
 #pragma unroll
@@ -305,12 +320,22 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
           }
         }
         if constexpr (READ_OUT) {
+          if constexpr (SPLIT == 2) {
+            float lower, upper;
+            lane_halves<32>(o, lower, upper);
+            o = lower + upper;
+          }
           const float nq = wave_sum(part);
           o = o / (fmaxf(fabsf(nq), bw_expf(-mn)) + 1e-6f);
         }
       }
       if constexpr (READ_OUT) {
-        if (live) a.out[(size_t)(first + t0 + t) * a.ldo + h * vdim + j] = o;
+        if constexpr (SPLIT == 2 && !GATES) {
+          float lower, upper;
+          lane_halves<32>(o, lower, upper);
+          o = lower + upper;
+        }
+        if (live && lane < COLS) a.out[(size_t)(first + t0 + t) * a.ldo + h * vdim + j] = o;
       }
     }
   }
@@ -326,8 +351,8 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
   if (PHASE == 3 && !leaves_state) return;
   if (live) {
 #pragma unroll
-    for (int d = 0; d < DPAD; ++d)
-      if (d < dim) S_out[(size_t)d * vdim + j] = Sreg[d];
+    for (int d = 0; d < DH; ++d)
+      if (dbase + d < dim) S_out[(size_t)(dbase + d) * vdim + j] = Sreg[d];
   }
   if (cb == 0 && (GATES || PHASE == 1)) {
 #pragma unroll
@@ -382,7 +407,8 @@ __global__ __launch_bounds__(256) void recurrence_scan_kernel(RecurArgs a, const
 
 template <int MODE, int PHASE>
 int launch_recurrence(const RecurArgs& a, int units, hipStream_t s) {
-  const dim3 grid((a.vdim + 63) / 64, a.heads, units), block(64);
+  const int cols = a.dim > 64 ? 32 : 64;      // (columns a wave: linear_recurrence_kernel's COLS)
+  const dim3 grid((a.vdim + cols - 1) / cols, a.heads, units), block(64);
   if (a.dim <= 16) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 16, PHASE>), grid, block, 0, s, a);
   else if (a.dim <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 32, PHASE>), grid, block, 0, s, a);
   else if (a.dim <= 64) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 64, PHASE>), grid, block, 0, s, a);

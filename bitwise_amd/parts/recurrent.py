@@ -26,8 +26,8 @@ from .base import Mixer, StateSpec, TensorSpec, register_mixer
 from .linear import Linear
 
 
-SCAN_CHUNK = 64          # rows of a chunk of a long portion
-SCAN_MIN_ROWS = 128      # portions from this many rows on run in three passes over chunks (shorter ones: one wave each)
+SCAN_CHUNK = 32          # rows of a chunk of a long portion
+SCAN_MIN_ROWS = 96       # portions from this many rows on run in three passes over chunks (shorter ones: one wave each)
 
 
 def _scan_plan(ctx):
