@@ -446,20 +446,32 @@ __global__ __launch_bounds__(64) void shared_key_attention_mfma_kernel(MfmaAttnA
       const int page = min(max(table[kj / ps], 0), a.num_pages - 1);
       krow[u] = kc + ((size_t)page * ps + kj % ps) * dk;
     }
+    // (where the values' runs of 4 keys lie: asked of the table together with the keys' pages)
+    const bf16_t* vrun[2][2];
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int x = 0; x < 2; ++x) {
+        const int c = min(kb0 + 32 * w + 16 * x + 4 * g, pmax & ~3);
+        vrun[w][x] = vt + (size_t)min(max(table[c / ps], 0), a.num_pages - 1) * dv * ps + c % ps;
+      }
     f32x4 st[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) st[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    for (int d1 = 8 * g; d1 < dkp; d1 += 128) {          // four steps of 32 elements: their 16 loads are in flight together
-      u32x4 kf[4][4], qf[4];
+    // KST steps of 32 elements at a time: their 4 KST loads are in flight together (a single token's piece of 64 keys
+    // is one block, and what it waits for is memory)
+    constexpr int KST = NDT <= 16 ? 10 : 6;
+    for (int d1 = 8 * g; d1 < dkp; d1 += 32 * KST) {
+      u32x4 kf[KST][4], qf[KST];
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) {
+      for (int s4 = 0; s4 < KST; ++s4) {
         const int d0 = d1 + 32 * s4;
         qf[s4] = d0 < dkp ? *reinterpret_cast<const u32x4*>(qs + n * qstride + d0) : (u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
         for (int u = 0; u < 4; ++u) kf[s4][u] = d0 < dk ? *reinterpret_cast<const u32x4*>(krow[u] + d0) : (u32x4){0u, 0u, 0u, 0u};
       }
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4)
+      for (int s4 = 0; s4 < KST; ++s4)
 #pragma unroll
         for (int u = 0; u < 4; ++u)
           st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[s4][u]), as_bf16x8(qf[s4]), st[u], 0, 0, 0);
@@ -499,9 +511,8 @@ __global__ __launch_bounds__(64) void shared_key_attention_mfma_kernel(MfmaAttnA
       const u32x4 pf = {pack_bf16x2(st[2 * w][0], st[2 * w][1]), pack_bf16x2(st[2 * w][2], st[2 * w][3]),
                         pack_bf16x2(st[2 * w + 1][0], st[2 * w + 1][1]), pack_bf16x2(st[2 * w + 1][2], st[2 * w + 1][3])};
       const int key0 = kb0 + 32 * w + 4 * g, key1 = key0 + 16;
-      const int c0 = min(key0, pmax & ~3), c1 = min(key1, pmax & ~3);
-      const bf16_t* b0 = vt + (size_t)min(max(table[c0 / ps], 0), a.num_pages - 1) * dv * ps + c0 % ps;
-      const bf16_t* b1 = vt + (size_t)min(max(table[c1 / ps], 0), a.num_pages - 1) * dv * ps + c1 % ps;
+      const bf16_t* b0 = vrun[w][0];
+      const bf16_t* b1 = vrun[w][1];
       uint32_t keep0[2] = {0xffffffffu, 0xffffffffu}, keep1[2] = {0xffffffffu, 0xffffffffu};
       if (ragged) {
 #pragma unroll

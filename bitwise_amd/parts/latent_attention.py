@@ -22,7 +22,7 @@ from .base import CacheSpec, Mixer, TensorSpec, lookup, register_mixer, POSITION
 from .linear import Linear
 
 ROWS_PER_PROMPT_TILE = 4        # the 32-bit kernel: 16 query vectors a workgroup, 4 rows x 4 heads or a single token's 16 heads
-MAX_SPLITS = 32                 # pieces a single token's keys are cut into at most (each a multiple of 64 keys)
+MAX_SPLITS = 64                 # pieces a single token's keys are cut into at most (each a multiple of 64 keys)
 
 
 def _tiles(ctx, rows_per_tile: int):
