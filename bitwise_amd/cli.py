@@ -32,6 +32,8 @@ def _engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--max-num-seqs", type=int, default=32, help="running requests at a time")
     p.add_argument("--no-prefix-caching", action="store_true")
     p.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    p.add_argument("--fast-portions", action="store_true",
+                   help="let mixers run long prompt portions in parallel passes where that changes the logits' last bits with the cut")
 
 
 def _model_options(p: argparse.ArgumentParser) -> None:
@@ -53,7 +55,8 @@ def _load_model(args, bw):
 def _config(args, bw):
     return bw.EngineConfig(num_blocks=args.num_blocks, max_batched_tokens=args.max_batched_tokens,
                            max_num_seqs=args.max_num_seqs, prefix_caching=not args.no_prefix_caching,
-                           block_size=args.block_size, dtype=args.dtype, use_graphs=not args.no_graphs)
+                           block_size=args.block_size, dtype=args.dtype, use_graphs=not args.no_graphs,
+                           exact_cuts=not args.fast_portions)
 
 
 def _sim(args, bw) -> int:

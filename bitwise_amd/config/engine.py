@@ -49,6 +49,10 @@ class EngineConfig:
     portion_align: int = 64          # a prompt portion that ends before its prompt does ends at a multiple of this many
                                      # tokens where the budget allows (whole pages and whole 64-key partitions: the
                                      # kernels' rows of 16 then never straddle a page); 1: cut exactly at the budget
+    exact_cuts: bool = True          # a position's logits do not depend on how its request was cut into steps, to the last bit.
+                                     # False: a mixer that can run a long prompt portion in parallel passes does so (the matrix
+                                     # memories' three passes over chunks, several times faster for long prompts); the logits
+                                     # then depend on the cut in their last bits
     fault: int = 0                   # a test-only bug (``Fault``) for the simulator to catch; 0: none
 
     def validate(self) -> None:

@@ -120,7 +120,7 @@ class GpuExecutor:
         max_logit_rows = min(config.max_num_seqs, config.max_batched_tokens)
         self.runner = ModelRunner(asm, self.storage, self.max_model_len, max_rows=config.max_batched_tokens,
                                   max_logit_rows=max_logit_rows, use_graphs=config.use_graphs,
-                                  decode_phases=config.decode_phases)
+                                  decode_phases=config.decode_phases, exact_cuts=config.exact_cuts)
         self.sampler = Sampler(rt.device, max_logit_rows)
         # two steps may be under way at a time (one being read back, one launched ahead): two sets of buffers
         self._flip = 0

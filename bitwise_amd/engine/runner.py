@@ -124,7 +124,8 @@ class ModelRunner:
     storage's caches.  It keeps nothing in the model, so several runners may share one."""
 
     def __init__(self, model: AssembledModel, storage: CacheStorage, max_model_len: int, max_rows: int = 256,
-                 max_logit_rows: Optional[int] = None, use_graphs: bool = True, decode_phases: bool = False):
+                 max_logit_rows: Optional[int] = None, use_graphs: bool = True, decode_phases: bool = False,
+                 exact_cuts: bool = True):
         self.model, self.storage = model, storage
         self.rt = model.rt
         self.use_graphs = bool(use_graphs) and model.graph_safe
@@ -140,6 +141,7 @@ class ModelRunner:
         self.max_model_len = min(int(max_model_len), model.spec.max_positions)
         self.ws = Workspace(model.rt.device, ws_rows, storage.page_size, ws_logit_rows,
                             max_table_width=(self.max_model_len + storage.page_size - 1) // storage.page_size)
+        self.ws.exact_cuts = bool(exact_cuts)
         self._graphs: Dict[int, tuple] = {}
         # decode_phases: captured decode steps of few rows in bfloat16 mode run their products as phases of a few
         # launches (ops.chain), if every part launches through ops: the words the phases meet in, and the word that

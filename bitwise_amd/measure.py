@@ -52,13 +52,13 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
 
 
 def make_engine(bw, model, batch: int, steps_total: int, dtype: str, context: int = CONTEXT, decode_phases: bool = False,
-                portion_align: int = 64):
+                portion_align: int = 64, exact_cuts: bool = True):
     block = 16
     per_request = context + steps_total + 2 * block
     cfg = bw.EngineConfig(num_blocks=batch * ((per_request + block - 1) // block) + 8, max_batched_tokens=2048,
                           max_num_seqs=max(batch, 1), prefix_caching=False, fingerprint_logits=False,
                           block_size=block, dtype=dtype, max_model_len=max(4096, context + 1024),
-                          decode_phases=decode_phases, portion_align=portion_align)
+                          decode_phases=decode_phases, portion_align=portion_align, exact_cuts=exact_cuts)
     return bw.Engine(model, None, cfg)
 
 
@@ -85,11 +85,12 @@ def time_decode(engine, torch, steps: int, warmup: int):
 
 
 
-def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float, tokens: int = PREFILL_TOKENS) -> dict:
+def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float, tokens: int = PREFILL_TOKENS,
+                    exact_cuts: bool = True) -> dict:
     """One prompt of ``tokens`` tokens (2,048 unless said otherwise) in one step (model, head for the last row,
     sampling): the median of six after two untimed ones (the shader clock takes some milliseconds of load to rise
     from its idle 2.1 GHz to 2.4); the best of the six is given beside it."""
-    engine = make_engine(bw, model, 1, 8, dtype)
+    engine = make_engine(bw, model, 1, 8, dtype, exact_cuts=exact_cuts)
     g = torch.Generator().manual_seed(99)
     times = []
     for _ in range(8):
@@ -219,7 +220,7 @@ def measure_qkv_row_orders(torch, cfg: dict, calls: int = 30) -> dict:
 
 
 def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: int, warmup: int,
-                   context: int = CONTEXT, decode_phases: bool = False, portion_align: int = 64) -> dict:
+                   context: int = CONTEXT, decode_phases: bool = False, portion_align: int = 64, exact_cuts: bool = True) -> dict:
     """``steps`` decode steps of ``batch`` requests that each hold a context of ``context`` tokens (2,048 unless
     said otherwise): tokens a second, and the bytes a step has to read (every weight once, the cache of the live
     requests) over its time."""
@@ -231,7 +232,7 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
     # a whole block)
     fill_steps = -(-batch * context // (2048 - batch - 64)) + 1
     new_tokens = steps + warmup + fill_steps + 8
-    eng = make_engine(bw, model, batch, new_tokens, dtype, context, decode_phases, portion_align)
+    eng = make_engine(bw, model, batch, new_tokens, dtype, context, decode_phases, portion_align, exact_cuts)
     fill(eng, bw, torch, batch, vocab_of(cfg), new_tokens, seed=batch, context=context)
     assert len(eng.sched.running) == batch
     secs = time_decode(eng, torch, steps, warmup)

@@ -164,9 +164,12 @@ class LatentAttention(Mixer):
             # Single tokens: the keys a token can have (what its block table spans) are cut into pieces of a multiple of
             # 64, at most MAX_SPLITS of them, a wave each; few tokens with long contexts still fill the chip.  The cut
             # depends on the table's width alone, which a captured step fixes.
+            # The pieces are joined in another order than a wave walks its blocks of keys, so a position's last bits would depend
+            # on whether it came alone or inside a portion: an engine that promises bits under any cut (Workspace.exact_cuts)
+            # keeps single tokens on one wave per 16 heads.
             span = table.shape[1] * ws.page_size
             kchunk = 64 * max(1, -(-span // (64 * MAX_SPLITS)))
-            nsplit = max(1, -(-span // kchunk))
+            nsplit = 1 if getattr(ws, "exact_cuts", True) else max(1, -(-span // kchunk))
             partial = None
             if nsplit > 1:
                 # (room for the most pieces, for the power of two from this step's single tokens up: a few sizes at most)

@@ -27,14 +27,15 @@ from .linear import Linear
 
 
 SCAN_CHUNK = 32          # rows of a chunk of a long portion
-SCAN_MIN_ROWS = 96       # portions from this many rows on run in three passes over chunks (shorter ones: one wave each)
+SCAN_MIN_ROWS = 96       # portions from this many rows on run in three passes over chunks (shorter ones: one wave each),
+                         # where the engine allows logits to depend on the cut in their last bits (Workspace.exact_cuts False)
 
 
 def _scan_plan(ctx):
     """Which requests of the step bring long portions, cut into chunks: (seq_rows for the others, their count, chunks,
     number of chunks, spans, number of spans), or None if every portion is short (a step of single tokens always is).  One
     plan a step, shared by its layers."""
-    if getattr(ctx, "one_row_per_request", False):
+    if getattr(ctx, "one_row_per_request", False) or getattr(ctx.ws, "exact_cuts", True):
         return None
 
     def make():

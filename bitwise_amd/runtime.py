@@ -60,6 +60,10 @@ class Workspace:
             raise ValueError("a workspace needs room for at least one row")
         if self.page_size < 1 or self.page_size & (self.page_size - 1):
             raise ValueError(f"page size must be a power of two, got {self.page_size}")
+        # True: a position's logits must not depend on how its request was cut into steps, to the last bit.  False lets a
+        # part that can run a long portion in parallel passes do so where that changes the last bits (its owner sets it:
+        # EngineConfig.exact_cuts)
+        self.exact_cuts = True
         self._buffers: Dict[Any, torch.Tensor] = {}
         self.notes: Dict[Any, Any] = {}       # what parts have worked out for this workspace (sizes of their scratch)
 

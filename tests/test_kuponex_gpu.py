@@ -188,11 +188,12 @@ def test_long_decoding(folders, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_portions_beside_short_ones(folders, dtype):
     """Portions long enough for the recurrences' three passes over chunks (whole, cut at and beside a chunk's edge), alone and
-    in one step with a short portion and a single token of other requests."""
+    in one step with a short portion and a single token of other requests; the engine that runs them allows logits to depend
+    on the cut in their last bits (``exact_cuts=False``).  With the default the cuttings agree bit for bit."""
     name = "wide"
     toks = tokens_for(name, 330, 31)
     want = plain(name, folders[name], toks, dtype)
-    rp = replayer(folders[name], dtype, 1024)
+    rp = replayer(folders[name], dtype, 1024, exact_cuts=False)
     for k, cuts in enumerate(([330], [129, 201], [128, 128, 74], [191, 130])):
         assert close(run_cut(rp, f"w{k}", toks, cuts), want, dtype), cuts
     small, one = tokens_for(name, 9, 32), tokens_for(name, 3, 33)
@@ -205,6 +206,9 @@ def test_long_portions_beside_short_ones(folders, dtype):
     lg = rp.step([{"id": "long", "tokens": toks[260:], "want": [0, 69]}, {"id": "small", "tokens": small[5:], "want": [3]}], ["long", "small", "one"])
     assert close(lg[:2], want[[260, 329]], dtype) and close(lg[2:], plain(name, folders[name], small, dtype)[8:], dtype)
     assert rp.manager.all_free()
+    exact = replayer(folders[name], dtype, 1024)
+    runs = [run_cut(exact, f"e{k}", toks, cuts) for k, cuts in enumerate(([330], [129, 201], [17, 300], [2] * 20))]
+    assert all(np.array_equal(runs[0], r) for r in runs[1:])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -246,6 +250,21 @@ def test_engine_preemption_recomputes_state(folders):
     for i, ref in zip(ids, solo):
         assert eng.result(i).tokens == ref.tokens and eng.result(i).logits_fingerprint == ref.logits_fingerprint
     assert eng.manager.all_free()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_randomized_scenarios_to_the_last_bit(gpu, dtype):
+    """The scenario simulator on the architecture's tiny model: page sizes, graphs, pools and budgets drawn per scenario,
+    every request against its solo run: no wrong token, no other logits (the default engine promises bits under any cut),
+    no page or slot lost; preemption happens on the way and restarts from zeroed state."""
+    from bitwise_amd.registry import ARCHITECTURES
+    from bitwise_amd.sim import Simulator
+
+    model = bw.Model.random(ARCHITECTURES["Kuponex"].tiny_config, 42, dtype, sigma=0.08)
+    tally = Simulator(model, dtype).run(16, seed=1)
+    print(tally.line(dtype))
+    assert tally.violations() == 0, "\n".join(tally.notes[:10])
+    assert tally.requests_compared > 40 and tally.preemptions > 0 and tally.prefix_hit_tokens == 0
 
 
 # ----------------------------------------------------------------------------- mechanisms made to matter
