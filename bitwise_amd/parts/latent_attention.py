@@ -4,7 +4,8 @@ part shared by all heads are cached; a head's key is [W_uk c | rotated part], it
 The scores are taken in the cache's own space: q_unrotated . (W_uk c) = (W_uk^T q_unrotated) . c, so a head's
 query becomes [W_uk^T q_unrotated | q_rotated] and one dot product with the cached vector is the score; the
 softmax-weighted sum of cached latents is projected to the head's values by W_uv afterwards.  The softmax has
-a sink: a learned score per head that joins the denominator, has no key and no value and is not scaled.
+a sink: one learned number per head that enters the denominator as exp(sink) beside the keys' terms (nothing is
+looked up for it, nothing is added to the output for it, and the score scale does not apply to it).
 
 Rotations, the latent's norm, scores and softmax weights are 32-bit in both modes; the cache holds the mode's
 activation dtype.

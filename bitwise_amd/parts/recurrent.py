@@ -7,8 +7,8 @@ projection added into the residual stream) and differ in the decay:
 * ``gla``: gated linear attention, a decay per key channel, alpha = sigmoid(z)^(1/tau) with z a low-rank
   projection of the input plus a bias; the read-out norm has one weight vector for all heads and the gate is SiLU.
 * ``mlstm``: the matrix memory of the xLSTM, scalar input and forget gates per head in the log domain, capped by
-  cap * tanh(. / cap), with a normaliser n and a running maximum m that starts at 0; the read-out is divided by
-  max(|n.q|, exp(-m)) + 1e-6, the norm weight spans all heads and the gate is a sigmoid.
+  cap * tanh(. / cap), with a normaliser n and a stabilising maximum m (a new request's m is 0, like the rest of its
+  state); the read-out is divided by max(|n.q|, exp(-m)) + 1e-6, the norm weight spans all heads and the gate is a sigmoid.
 
 The state, the gates and everything between the projections and the read-out are 32-bit in both modes; the
 projections' sums arrive as 32-bit values and are not rounded on the way.

@@ -52,6 +52,8 @@ CONFIGS = {
     "only_mlstm": config(48, 61, 1e-5, [mlstm(3, 8, 20, 6.0, None)]),
     "only_latent": config(48, 61, 1e-5, [latent(3, 8, 8, 12, 24, 0.3, 300.0, 8, None)]),
     "only_latent_odd": config(48, 61, 1e-5, [latent(5, 6, 6, 10, 21, 0.3, 300.0, 6, None)]),      # a key vector that is no multiple of 8
+    # more heads than a wave's 16 query vectors (a second, partly filled group), tiny heads; eps that matters
+    "many_heads": config(40, 67, 1e-2, [latent(18, 4, 4, 4, 12, 0.5, 50.0, 4, 48), gla(5, 8, 4, 2.0, 2, None), mlstm(6, 4, 12, 3.0, 32)]),
     # everything together, sizes all different, a partly rotated key part, a layer without feed-forward, one head
     "mixed": config(64, 131, 1e-5, [mlstm(2, 16, 24, 8.0, 96), latent(3, 8, 8, 20, 24, 0.2, 500.0, 4, 80),
                                      gla(4, 8, 8, 4.0, 3, None), latent(1, 16, 4, 8, 12, 0.25, 10000.0, 4, 72),
