@@ -17,10 +17,11 @@ pytestmark = pytest.mark.gpu
 
 # float32: a row now and then sits where a head's read-out nearly cancels and the 32-bit sums' last bits show (a few 1e-5); the
 # bulk is held to 5e-6.
-# bfloat16: against the plain model rounded at the engine's rounding points; what is left are roundings that fall the
-# other way because 32-bit sums differ from exact ones in their last bits (a row now and then, so the bulk is held to
-# half of the limit)
-TOL = {"float32": 1e-4, "bfloat16": 2e-2}
+# bfloat16: against the plain model rounded at the engine's rounding points; what is left are the queries and softmax
+# weights that the matrix-core attention rounds on their way into its products, and roundings that fall the other way
+# because 32-bit sums differ from exact ones in their last bits (some 5e-3 a row in a model of several layers, a few
+# 1e-2 in a row now and then; a mechanism that is wrong moves a row by its own size and shows in 32-bit first)
+TOL = {"float32": 1e-4, "bfloat16": 5e-2}
 TYPICAL = {"float32": 5e-6, "bfloat16": 1e-2}
 RND = {"float32": pk.identity, "bfloat16": pk.round_bf16}
 SIGMA = 0.15
@@ -62,7 +63,7 @@ CONFIGS = {
     "wide": config(96, 77, 1e-6, [gla(2, 40, 72, 8.0, 6, 120), mlstm(2, 72, 40, 12.0, 64),
                                    latent(5, 12, 16, 24, 72, 0.15, 2000.0, 16, 104), mlstm(1, 8, 136, 20.0, None)]),
 }
-SEEDS = {name: i + 11 for i, name in enumerate(CONFIGS)}
+SEEDS = {"only_gla": 11, "only_mlstm": 12, "only_latent": 13, "only_latent_odd": 14, "mixed": 15, "wide": 16, "many_heads": 17}
 
 
 @pytest.fixture(scope="module")
