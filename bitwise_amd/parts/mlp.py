@@ -90,12 +90,22 @@ class GeGLU(SwiGLU):
     default_names = ("gate", "up", "down")
 
     def forward_with_norm(self, ctx, x, norm, residual) -> bool:
-        return False
+        """Decode steps of few rows: the norm rides in the stacked product (the bits of norm, then product)."""
+        from .norm import RMSNorm
+        ws, rows = ctx.ws, ctx.rows
+        if not (self.rt.bf16 and type(norm) is RMSNorm and self.gate_up.mfma and ops.can_fuse_norm(rows, self.gate_up.weight, x)):
+            return False
+        gu = ws.buffer("gate_up", 2 * self.inter, torch.float32)
+        ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.gate_up.weight, gu, rows, ops.EPI_F32)
+        self._gate_and_down(ctx, gu, residual)
+        return True
+
+    def _gate_and_down(self, ctx, gu, residual) -> None:
+        act = ctx.ws.buffer("mlp_h", self.inter, self.rt.act_dtype)
+        ops.glu(gu, act, ctx.rows, self.act)
+        self.down.add_into(ctx.ws, act, residual, ctx.rows)
 
     def forward(self, ctx, h, residual) -> None:
-        ws, rows = ctx.ws, ctx.rows
-        gu = ws.buffer("gate_up", 2 * self.inter, torch.float32)
-        self.gate_up.store(ws, h, gu, rows)
-        act = ws.buffer("mlp_h", self.inter, self.rt.act_dtype)
-        ops.glu(gu, act, rows, self.act)
-        self.down.add_into(ws, act, residual, rows)
+        gu = ctx.ws.buffer("gate_up", 2 * self.inter, torch.float32)
+        self.gate_up.store(ctx.ws, h, gu, ctx.rows)
+        self._gate_and_down(ctx, gu, residual)
