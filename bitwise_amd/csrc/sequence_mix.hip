@@ -135,6 +135,21 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict
 
 enum { RECUR_DECAY_PER_CHANNEL = 0, RECUR_SCALAR_GATES = 1 };
 
+// The sum over the lanes l, l + 64/SPLIT, ... that hold the parts of one column (every one of them gets it).
+template <int SPLIT>
+__device__ __forceinline__ float join_parts(float v) {
+  if constexpr (SPLIT >= 2) {
+    float lower, upper;
+    lane_halves<32>(v, lower, upper);
+    v = lower + upper;
+    if constexpr (SPLIT == 4) {
+      lane_halves<16>(v, lower, upper);
+      v = lower + upper;
+    }
+  }
+  return v;
+}
+
 struct RecurArgs {
   const float* proj;       // [rows, ldp]: the rows' stacked projections
   int ldp, q_off, k_off, v_off;
@@ -160,7 +175,7 @@ struct RecurArgs {
   float* start;            // per chunk: the state it starts from (S; scalar gates: n, m)
 };
 
-// One wave per (request, head, block of 64 value columns; 32 for heads of more than 64 key channels).  Lane j keeps column j of the head's state matrix in
+// One wave per (request, head, block of 64, 32 or 16 value columns: see SPLIT).  Lane j keeps column j of the head's state matrix in
 // registers (one element per key channel), so the read-out S^T q needs no exchange between lanes; the tokens' q, k and
 // decays come through LDS in chunks of RC tokens and are read from there by all lanes at once.
 //
@@ -176,22 +191,25 @@ struct RecurArgs {
 // chunk from there with the read-out, and the request's last chunk leaves the state in the slot.  PHASE 0 is the whole
 // portion by one wave.  The passes differ from PHASE 0 by the rounding of the scan's sums only.
 #define RC 16
+#define RW 4             // waves of a workgroup: neighbouring column blocks of one head, which share the staged tokens
 template <int MODE, int DPAD, int PHASE>
-__global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
+__global__ __launch_bounds__(64 * RW) void linear_recurrence_kernel(RecurArgs a) {
   constexpr bool GATES = MODE == RECUR_SCALAR_GATES;
   constexpr int NN = (DPAD + 63) / 64;
   constexpr bool READ_OUT = PHASE != 1;
-  // heads of 128 key channels and more: a column's channels are split over two lanes (lane l and l + 32 hold the two halves
-  // of column l mod 32), so that a lane's part of the state fits its registers; the halves' read-outs are added lower + upper
-  constexpr int SPLIT = DPAD >= 128 ? 2 : 1;
+  // A column's key channels are split over SPLIT lanes (lane l, l + COLS, ... hold consecutive parts of column l mod COLS): a
+  // lane's part of the state is at most 64 registers and a token costs a lane DPAD / SPLIT steps, so a head has more and
+  // shorter waves.  The parts' read-outs are added by the swaps of the wave's halves and quarters, in one order whatever
+  // runs the head (a single token, a portion, a chunk): the split depends on the head's size alone.
+  constexpr int SPLIT = DPAD >= 64 ? 4 : (DPAD >= 32 ? 2 : 1);
   constexpr int DH = DPAD / SPLIT, COLS = 64 / SPLIT;
   __shared__ float qs[RC][DPAD];
   __shared__ float ks[RC][DPAD];
   __shared__ float as[GATES ? 1 : RC][GATES ? 1 : DPAD];
   __shared__ float gi[RC], gf[RC];
-  __shared__ float vs[RC][64];
-  const int lane = threadIdx.x;
-  const int cb = blockIdx.x, h = blockIdx.y;
+  __shared__ float vs[RW][RC][64];
+  const int lane = threadIdx.x & 63, wv = wave_index();
+  const int cb = blockIdx.x * RW + wv, h = blockIdx.y;
   const int dim = a.dim, vdim = a.vdim;
   const size_t rec = (size_t)dim * vdim + dim + 2;
   int first, count, slot;
@@ -245,11 +263,11 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
     const int tc = min(RC, count - t0);
     __syncthreads();
     // eight elements a lane at a time: their loads are all asked for before the first is used
-    for (int e0 = 0; e0 < tc * DPAD; e0 += 64 * 8) {
+    for (int e0 = 0; e0 < tc * DPAD; e0 += 64 * RW * 8) {
       float qv[8], kv[8], zv[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        const int e = e0 + 64 * u + lane;
+        const int e = e0 + 64 * RW * u + (int)threadIdx.x;
         const int t = e / DPAD, d = e % DPAD;
         const bool in = e < tc * DPAD && d < dim;
         const size_t row = (size_t)(first + t0 + min(t, tc - 1));
@@ -260,7 +278,7 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        const int e = e0 + 64 * u + lane;
+        const int e = e0 + 64 * RW * u + (int)threadIdx.x;
         if (e >= tc * DPAD) continue;
         const int t = e / DPAD, d = e % DPAD;
         qs[t][d] = qv[u] * a.qscale;
@@ -269,7 +287,7 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
       }
     }
     if constexpr (GATES) {
-      if (lane < tc) {
+      if (wv == 0 && lane < tc) {
         const float* pr = a.proj + (size_t)(first + t0 + lane) * a.ldp;
         const float cap = a.param;
         gi[lane] = cap * tanhf((pr[a.gate_off + h] + a.bias[h]) / cap);
@@ -280,13 +298,13 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
     if (lane < COLS) {
 #pragma unroll
       for (int t = 0; t < RC; ++t)
-        vs[t][col] = (live && t < tc) ? a.proj[(size_t)(first + t0 + t) * a.ldp + a.v_off + h * vdim + j] : 0.0f;
+        vs[wv][t][col] = (live && t < tc) ? a.proj[(size_t)(first + t0 + t) * a.ldp + a.v_off + h * vdim + j] : 0.0f;
     }
     __syncthreads();
     for (int t = 0; t < tc; ++t) {
       float o = 0.0f;
       if constexpr (!GATES) {
-        const float v = vs[t][col];
+        const float v = vs[wv][t][col];
 #pragma unroll
         for (int d = 0; d < DH; ++d) {
           Sreg[d] = fmaf(as[t][dbase + d], Sreg[d], ks[t][dbase + d] * v);
@@ -304,7 +322,7 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
         const float ib = bw_expf(ig - mn);
         m = mn;
         fsum += fg;
-        const float bv = ib * vs[t][col];
+        const float bv = ib * vs[wv][t][col];
 #pragma unroll
         for (int d = 0; d < DH; ++d) {
           Sreg[d] = fmaf(fa, Sreg[d], ks[t][dbase + d] * bv);
@@ -320,21 +338,13 @@ __global__ __launch_bounds__(64) void linear_recurrence_kernel(RecurArgs a) {
           }
         }
         if constexpr (READ_OUT) {
-          if constexpr (SPLIT == 2) {
-            float lower, upper;
-            lane_halves<32>(o, lower, upper);
-            o = lower + upper;
-          }
+          o = join_parts<SPLIT>(o);
           const float nq = wave_sum(part);
           o = o / (fmaxf(fabsf(nq), bw_expf(-mn)) + 1e-6f);
         }
       }
       if constexpr (READ_OUT) {
-        if constexpr (SPLIT == 2 && !GATES) {
-          float lower, upper;
-          lane_halves<32>(o, lower, upper);
-          o = lower + upper;
-        }
+        if constexpr (!GATES) o = join_parts<SPLIT>(o);
         if (live && lane < COLS) a.out[(size_t)(first + t0 + t) * a.ldo + h * vdim + j] = o;
       }
     }
@@ -407,8 +417,8 @@ __global__ __launch_bounds__(256) void recurrence_scan_kernel(RecurArgs a, const
 
 template <int MODE, int PHASE>
 int launch_recurrence(const RecurArgs& a, int units, hipStream_t s) {
-  const int cols = a.dim > 64 ? 32 : 64;      // (columns a wave: linear_recurrence_kernel's COLS)
-  const dim3 grid((a.vdim + cols - 1) / cols, a.heads, units), block(64);
+  const int cols = a.dim > 32 ? 16 : (a.dim > 16 ? 32 : 64);      // (columns a wave: linear_recurrence_kernel's COLS)
+  const dim3 grid((a.vdim + RW * cols - 1) / (RW * cols), a.heads, units), block(64 * RW);
   if (a.dim <= 16) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 16, PHASE>), grid, block, 0, s, a);
   else if (a.dim <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 32, PHASE>), grid, block, 0, s, a);
   else if (a.dim <= 64) hipLaunchKernelGGL((linear_recurrence_kernel<MODE, 64, PHASE>), grid, block, 0, s, a);
