@@ -69,7 +69,6 @@ class _MatrixMemoryMixer(Mixer):
     mode = -1
     gate_kind = ops.GATE_SIGMOID
     per_head_norm_weight = True
-    stacked: Tuple[str, ...] = ()                # the projections of the input that are stacked into one product
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
