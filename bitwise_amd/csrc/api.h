@@ -48,16 +48,16 @@ int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, void* q_out
 int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, const int32_t* row_seq,
                      const int32_t* block_table, int table_stride, const float* k_cache, const float* v_cache,
                      float* out, int out_stride, int rows, int heads, int kv_heads, int head_dim, int page_size,
-                     int window, float scale, void* stream);
+                     int window, float scale, const float* sink, void* stream);
 int bw_attention_f32_tiles(const float* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                            int table_stride, const int32_t* tiles, int num_tiles, int tiled, const float* k_cache,
                            const float* v_cache, float* out, int out_stride, int heads, int kv_heads, int head_dim,
-                           int page_size, int window, float scale, void* stream);
+                           int page_size, int window, float scale, const float* sink, void* stream);
 int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                       int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
                       const void* v_cache, int num_pages, void* out, int out_stride, int heads, int kv_heads,
                       int head_dim, int page_size, int window, float scale, int decode, float* scratch,
-                      long long scratch_floats, int32_t* counters, int num_counters, void* stream);
+                      long long scratch_floats, int32_t* counters, int num_counters, const float* sink, void* stream);
 int bw_attention_decode_scratch(int num_tiles, int heads, int kv_heads, int head_dim, int table_stride,
                                 int page_size, long long* scratch_floats, int* counters);
 int bw_attention_fold_group_tiles(int head_dim);
@@ -124,4 +124,35 @@ int bw_shared_key_attention_mfma(const void* q, int ldq, const int32_t* position
                                  const void* latent_t, int num_pages, const float* sink, float* out, int ldo, int heads,
                                  int dk, int dv, int page_size, int window, float scale, int heads_per_group, int nsplit,
                                  int kchunk, float* partial, long long partial_floats, void* stream);
+// Mixers that convolve their projections over a few tokens, gate their outputs or carry a gated recurrence per channel,
+// and row operations of layers whose norm sits behind the sublayer (gated_mix.hip).  sink (the attention entry points
+// above): a score per head that joins the softmax's denominator and has no value, or null.
+int bw_causal_conv(const float* x, int ldx, const void* w, const void* bias, int w_is_bf16, int taps, int channels,
+                   float* state, long long state_ld, const int32_t* seq_rows, const int32_t* slots,
+                   const int32_t* positions, int nseq, int max_seq_rows, float* out, int ldo, void* stream);
+int bw_pair_rope_unit(const float* src, int lds, const int32_t* positions, const int32_t* row_seq,
+                      const int32_t* block_table, int table_stride, const float* cos_table, const float* sin_table,
+                      void* q_out, void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads,
+                      int dim, int vdim, int hd, int rot, int page_size, int unit_norm, float eps, int has_kv,
+                      int write_cache, void* stream);
+int bw_gate_mul(const void* av, int a_is_bf16, int lda, int hd, const float* g, int ldg, void* out, int out_is_bf16,
+                int ldo, int rows, int heads, int vdim, void* stream);
+int bw_rglru_scan(const float* y, int ldy, const float* u, int ldu, const float* gates, int ldg, const float* ra_bias,
+                  const float* ri_bias, const float* decay, float* state, long long state_ld, void* out,
+                  int out_is_bf16, int ldo, const int32_t* seq_rows, const int32_t* slots, const int32_t* positions,
+                  int nseq, int channels, int bs, void* stream);
+int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, int rows, int dim, float eps,
+                void* stream);
+int bw_softcap(float* x, int ld, int rows, int cols, float cap, void* stream);
+// A feed-forward of routed experts (moe.hip).
+int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
+                 float* wts, void* stream);
+int bw_moe_max_tiles(int slots, int experts);
+int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* sorted, int32_t* place, int32_t* tiles,
+                int32_t* meta, int32_t* rank, void* stream);
+int bw_moe_experts(const void* x, int x_is_bf16, int ldx, const void* w, int w_is_bf16, void* out, int ldo,
+                   const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int max_tiles, int top, int K,
+                   int N, int gate_up, float limit, float alpha, int round_out, void* stream);
+int bw_moe_combine(const float* y, int ldy, const int32_t* place, const float* wts, int top, float* out, int ldo,
+                   int rows, int width, int accumulate, void* stream);
 }

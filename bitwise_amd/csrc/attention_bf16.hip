@@ -46,7 +46,13 @@ struct AttnBf16Args {
   bf16_t* out;                // [rows, out_stride]
   int heads, kv_heads, page_size, page_shift, num_pages, table_stride, q_stride, out_stride, window, hpt, nsub, num_tiles;
   float scale_log2;           // softmax scale times log2(e)
+  const float* sink;          // [heads] or null: a score per head that joins the softmax's denominator and has no value
 };
+
+// What the sink adds to a query's folded sum l, whose terms are taken against the folded maximum m (base-2 domain).
+__device__ __forceinline__ float sink_term(const AttnBf16Args& a, int head, float m) {
+  return a.sink != nullptr ? __builtin_amdgcn_exp2f(fminf(a.sink[head] * 1.44269504088896340736f - m, 120.0f)) : 0.0f;
+}
 
 // What the lanes of a wave share for one group of tiles: sequence, kv head, key range.
 struct GroupCtx {
@@ -673,7 +679,7 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
     if (tc[t].pos_c < 0) continue;
-    const float inv = 1.0f / l[t];
+    const float inv = 1.0f / (l[t] + sink_term(a, tc[t].head_c, m[t]));
     bf16_t* dst = a.out + (size_t)tc[t].row_c * a.out_stride + (size_t)tc[t].head_c * HD;
 #pragma unroll
     for (int dt = 0; dt < NT; ++dt) {
@@ -848,7 +854,7 @@ __device__ __forceinline__ void decode_fold_pass(const AttnBf16Args& a, const Gr
   for (int e = threadIdx.x; e < elems; e += THREADS) {
     const int col = e / HD, d = e % HD;
     if (gc.sub * a.hpt + col >= group) continue;       // columns of a one-token tile: column c is head sub*hpt + c of the kv head's group
-    const float inv = 1.0f / lds.lsum[col];
+    const float inv = 1.0f / (lds.lsum[col] + sink_term(a, gc.kvh * group + gc.sub * a.hpt + col, m_after[col]));
     a.out[(size_t)row * a.out_stride + (size_t)(gc.kvh * group + gc.sub * a.hpt + col) * HD + d] = f32_to_bf16(lds.state[e] * inv);
   }
 }
@@ -1119,7 +1125,7 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
                                  const void* v_cache, int num_pages, void* out, int out_stride, int heads,
                                  int kv_heads, int head_dim, int page_size, int window, float scale, int decode,
                                  float* scratch, long long scratch_floats, int32_t* counters, int num_counters,
-                                 void* stream) {
+                                 const float* sink, void* stream) {
   if (num_tiles <= 0) return 0;
   if (num_pages <= 0) return -2;
   if (kv_heads <= 0 || heads % kv_heads) return -2;
@@ -1137,6 +1143,7 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
   a.hpt = group < 16 ? group : 16;
   a.nsub = (group + a.hpt - 1) / a.hpt;
   a.num_tiles = num_tiles;
+  a.sink = sink;
   if (!(scale > 0.0f)) return -2;                // the maximum is taken before the scaling
   a.scale_log2 = scale * 1.44269504088896340736f;
   if (kv_heads * a.nsub > 65535) return -2;

@@ -25,7 +25,14 @@ struct AttnF32Args {
   float scale;
   int page_shift;            // log2 of the page size, or -1 if it is no power of two
   const int32_t* tiles;      // [tiles][4] = row0, tokens, seq, 0 (consecutive rows of one sequence); null: a row a workgroup
+  const float* sink;         // [heads] or null: a score per head that joins the softmax's denominator and has no value
 };
+
+// What the sink adds to a query's sum of exponentials taken against the maximum mx of its keys' scores (the keys'
+// terms stay as they are; a sink far above every key gives a huge term and an output of zero).
+__device__ __forceinline__ float sink_term(const AttnF32Args& a, int h, float mx) {
+  return a.sink != nullptr ? bw_expf(fminf(a.sink[h] - mx, 80.0f)) : 0.0f;
+}
 
 // A key's row in registers.
 template <int HD>
@@ -394,7 +401,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
       buf ^= 1;
     }
   }
-  if (tid < HD) a.out[(size_t)row * a.out_stride + (size_t)h * HD + tid] = acc * (1.0f / sum);
+  if (tid < HD) a.out[(size_t)row * a.out_stride + (size_t)h * HD + tid] = acc * (1.0f / (sum + sink_term(a, h, mx)));
 }
 
 // Prompt portions: a workgroup per tile of up to 16 consecutive rows of one sequence and head, so that a chunk of
@@ -542,7 +549,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_tile_kernel(AttnF
     }
   }
   if (pos_q >= 0) {
-    const float inv = 1.0f / sum;
+    const float inv = 1.0f / (sum + sink_term(a, h, mx));
     float* o = a.out + (size_t)my_row * a.out_stride + (size_t)h * HD + kl;
 #pragma unroll
     for (int u = 0; u < ND; ++u) o[16 * u] = acc[u] * inv;
@@ -866,7 +873,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #undef ATT_VALUES
   }
   // out[q][d] = acc[q][d] * (1 / sum[q]): register r of block b is query 8 (r / 4) + 4 h2 + r % 4, element 64 nb + 32 b + col
-  const float inv = 1.0f / sum;
+  const float inv = 1.0f / (sum + sink_term(a, h, mx));
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int q = 8 * (r >> 2) + key_of_reg + (r & 3);
@@ -940,11 +947,11 @@ static int attention_f32_dispatch(const AttnF32Args& a, int items, int tiled, hi
 extern "C" int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, const int32_t* row_seq,
                                 const int32_t* block_table, int table_stride, const float* k_cache,
                                 const float* v_cache, float* out, int out_stride, int rows, int heads,
-                                int kv_heads, int head_dim, int page_size, int window, float scale, void* stream) {
+                                int kv_heads, int head_dim, int page_size, int window, float scale, const float* sink, void* stream) {
   if (rows <= 0) return 0;
   AttnF32Args a{q, positions, row_seq, block_table, k_cache, v_cache, out, rows, heads, kv_heads, head_dim,
                 page_size, table_stride, q_stride, out_stride, window, scale,
-                (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1, nullptr};
+                (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1, nullptr, sink};
   return attention_f32_dispatch(a, rows, 0, (hipStream_t)stream);
 }
 
@@ -955,11 +962,12 @@ extern "C" int bw_attention_f32(const float* q, int q_stride, const int32_t* pos
 extern "C" int bw_attention_f32_tiles(const float* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                                       int table_stride, const int32_t* tiles, int num_tiles, int tiled,
                                       const float* k_cache, const float* v_cache, float* out, int out_stride, int heads,
-                                      int kv_heads, int head_dim, int page_size, int window, float scale, void* stream) {
+                                      int kv_heads, int head_dim, int page_size, int window, float scale, const float* sink,
+                                      void* stream) {
   if (num_tiles <= 0) return 0;
   if (tiles == nullptr) return -2;
   AttnF32Args a{q, positions, nullptr, block_table, k_cache, v_cache, out, 0, heads, kv_heads, head_dim,
                 page_size, table_stride, q_stride, out_stride, window, scale,
-                (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1, tiles};
+                (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1, tiles, sink};
   return attention_f32_dispatch(a, num_tiles, tiled, (hipStream_t)stream);
 }

@@ -23,7 +23,7 @@ from typing import List, Optional
 
 HERE = Path(__file__).resolve().parent
 SOURCES = ["elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_f32.hip", "attention_bf16.hip",
-           "fused_decode.hip", "sampling.hip", "sequence_mix.hip", "latent_attention.hip"]
+           "fused_decode.hip", "sampling.hip", "sequence_mix.hip", "latent_attention.hip", "gated_mix.hip", "moe.hip"]
 HEADERS = ["common.h", "api.h", "layout.h", "gemm_bf16_skinny.h", "gemm_bf16_tiles.h", "gemm_bf16_rows.h",
            "gemm_bf16_phases.h"]
 LIB_NAME = "libbitwise_hip.so"

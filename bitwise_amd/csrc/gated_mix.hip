@@ -1,0 +1,379 @@
+// Kernels around mixers that convolve their projections over a few tokens, gate their outputs, or carry a
+// gated linear recurrence per channel; and the small row operations of a layer whose norm sits behind the sublayer.
+//
+//   causal_conv:   y_t[c] = sum_j w[c][j] * u_(t - taps + 1 + j)[c] (+ bias[c]); the last taps-1 inputs of every request
+//                  live in its state slot, so a portion of any length continues where the last one stopped
+//   pair_rope_unit: rotation of neighbouring pairs (2i, 2i+1) of the first rot elements of each head at the row's
+//                  position, optional division by the head's root mean square, the cache write (keys and values padded
+//                  with zeros to the cache's head size) and the queries' copy
+//   gate_mul:      out = a * sigmoid(g), heads compacted from the attention's head size to the value size
+//   rglru_scan:    S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t with a_t = exp(c r_t), r and i sigmoids of block-diagonal
+//                  projections of u; out = S_t * gelu_tanh(y_t)
+//   norm_add:      x += y / sqrt(mean(y^2) + eps) * w
+//   softcap:       x = cap * tanh(x / cap)
+//
+// All arithmetic is 32-bit; only stores into a bfloat16 buffer round.  A request without rows, with a negative slot or
+// a negative first position is padding and leaves its state alone.
+#include <math.h>
+
+#include "common.h"
+#include "api.h"
+
+template <typename T> __device__ __forceinline__ float gm_load(const T* p);
+template <> __device__ __forceinline__ float gm_load<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float gm_load<bf16_t>(const bf16_t* p) { return bf16_to_f32(*p); }
+__device__ __forceinline__ void gm_store(float* p, float v) { *p = v; }
+__device__ __forceinline__ void gm_store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+__device__ __forceinline__ float gm_sigmoid(float x) { return 1.0f / (1.0f + bw_expf(-x)); }
+
+// ------------------------------------------------------------------------------ short causal convolution
+
+#define CONV_CHUNK 32
+#define CONV_MAX_TAPS 8
+
+struct ConvArgs {
+  const float* x;        // [rows, ldx]: channel c at column c
+  const void* w;         // [channels, taps]
+  const void* bias;      // [channels] or null
+  float* state;          // [slots, state_ld]: [taps - 1][channels] at the pointer, oldest first
+  float* out;            // [rows, ldo]
+  const int32_t* seq_rows;
+  const int32_t* slots;
+  const int32_t* positions;
+  long long state_ld;
+  int ldx, ldo, channels;
+};
+
+template <int TAPS, typename WT>
+__global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
+  constexpr int P = TAPS > 1 ? TAPS - 1 : 1;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int seq = blockIdx.y, t0 = blockIdx.z * CONV_CHUNK;
+  const int first = a.seq_rows[2 * seq], n = a.seq_rows[2 * seq + 1], slot = a.slots[seq];
+  if (c >= a.channels || n <= 0 || slot < 0 || t0 >= n || a.positions[first] < 0) return;
+  const int t1 = min(n, t0 + CONV_CHUNK);
+  float w[TAPS];
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) w[j] = gm_load(reinterpret_cast<const WT*>(a.w) + (size_t)c * TAPS + j);
+  const float bias = a.bias != nullptr ? gm_load(reinterpret_cast<const WT*>(a.bias) + c) : 0.0f;
+  float* st = a.state + (size_t)slot * a.state_ld + c;
+  const float* x = a.x + (size_t)first * a.ldx + c;
+  // only the request's first chunk reaches back before the portion, and only its threads touch the slot
+  float old[P];
+#pragma unroll
+  for (int j = 0; j < P; ++j) old[j] = (TAPS > 1 && t0 == 0) ? st[(size_t)j * a.channels] : 0.0f;
+  float win[P];
+#pragma unroll
+  for (int j = 0; j < P; ++j) {
+    const int idx = t0 - (TAPS - 1) + j;
+    win[j] = idx >= 0 ? x[(size_t)idx * a.ldx] : old[(TAPS - 1 + idx) < 0 ? 0 : (TAPS - 1 + idx)];
+  }
+  float* o = a.out + (size_t)first * a.ldo + c;
+  for (int t = t0; t < t1; ++t) {
+    const float cur = x[(size_t)t * a.ldx];
+    float acc = 0.0f;
+    if constexpr (TAPS > 1) {
+#pragma unroll
+      for (int j = 0; j < TAPS - 1; ++j) acc = fmaf(w[j], win[j], acc);
+    }
+    acc = fmaf(w[TAPS - 1], cur, acc);
+    if (a.bias != nullptr) acc += bias;
+    o[(size_t)t * a.ldo] = acc;
+    if constexpr (TAPS > 1) {
+#pragma unroll
+      for (int j = 0; j + 1 < TAPS - 1; ++j) win[j] = win[j + 1];
+      win[TAPS - 2] = cur;
+    }
+  }
+  if (TAPS > 1 && t0 == 0) {
+#pragma unroll
+    for (int j = 0; j < TAPS - 1; ++j) {
+      const int idx = n - (TAPS - 1) + j;
+      float v = 0.0f;
+      if (idx >= 0) v = x[(size_t)idx * a.ldx];
+      else {
+#pragma unroll
+        for (int q = 0; q < P; ++q) v = (q == TAPS - 1 + idx) ? old[q] : v;
+      }
+      st[(size_t)j * a.channels] = v;
+    }
+  }
+}
+
+template <typename WT>
+static int conv_launch(const ConvArgs& a, int taps, dim3 grid, hipStream_t s) {
+  switch (taps) {
+#define CONV_CASE(T) case T: hipLaunchKernelGGL((causal_conv_kernel<T, WT>), grid, dim3(256), 0, s, a); break;
+    CONV_CASE(1) CONV_CASE(2) CONV_CASE(3) CONV_CASE(4) CONV_CASE(5) CONV_CASE(6) CONV_CASE(7) CONV_CASE(8)
+#undef CONV_CASE
+    default: return -2;
+  }
+  return BW_LAUNCH_CHECK();
+}
+
+extern "C" int bw_causal_conv(const float* x, int ldx, const void* w, const void* bias, int w_is_bf16, int taps, int channels,
+                              float* state, long long state_ld, const int32_t* seq_rows, const int32_t* slots,
+                              const int32_t* positions, int nseq, int max_seq_rows, float* out, int ldo, void* stream) {
+  if (nseq <= 0 || channels <= 0 || max_seq_rows <= 0) return 0;
+  if (taps < 1 || taps > CONV_MAX_TAPS || (taps > 1 && state == nullptr)) return -2;
+  ConvArgs a{x, w, bias, state, out, seq_rows, slots, positions, state_ld, ldx, ldo, channels};
+  const dim3 grid((channels + 255) / 256, nseq, (max_seq_rows + CONV_CHUNK - 1) / CONV_CHUNK);
+  if (grid.y > 65535 || grid.z > 65535) return -2;
+  return w_is_bf16 ? conv_launch<bf16_t>(a, taps, grid, (hipStream_t)stream) : conv_launch<float>(a, taps, grid, (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------------------ pair rotation, unit norm, cache write
+
+struct PairRopeArgs {
+  const float* src;            // [rows, lds]: q heads (dim each), then k heads (dim each), then v heads (vdim each)
+  const int32_t* positions;
+  const int32_t* row_seq;
+  const int32_t* block_table;
+  const float* cos_table;      // [positions, rot / 2]
+  const float* sin_table;
+  void* q_out;                 // [rows, heads * hd]
+  void* k_cache;
+  void* v_cache;
+  int lds, rows, heads, kv_heads, dim, vdim, hd, rot, page_size, table_stride, unit_norm, has_kv, write_cache;
+  float eps;
+};
+
+// A wave a (row, head): q heads, then k heads, then v heads.  Lane l owns the pairs l, l + 64, ...
+template <typename T>
+__global__ __launch_bounds__(256) void pair_rope_unit_kernel(PairRopeArgs a) {
+  const int per_row = a.heads + (a.has_kv ? 2 * a.kv_heads : 0);
+  const int item = blockIdx.x * 4 + wave_index();
+  if (item >= a.rows * per_row) return;
+  const int row = item / per_row, hh = item % per_row, lane = threadIdx.x & 63;
+  const int pos = a.positions[row];
+  if (pos < 0) return;
+  const bool is_q = hh < a.heads, is_k = !is_q && hh < a.heads + a.kv_heads;
+  if (!is_q && !a.write_cache) return;
+  const int page = a.block_table[(size_t)a.row_seq[row] * a.table_stride + pos / a.page_size];
+  const int slot = pos % a.page_size;
+  if (!is_q && !is_k) {
+    // values: as they are, padded with zeros to the cache's head size
+    const int h = hh - a.heads - a.kv_heads;
+    const float* v = a.src + (size_t)row * a.lds + (size_t)(a.heads + a.kv_heads) * a.dim + (size_t)h * a.vdim;
+    T* vc = reinterpret_cast<T*>(a.v_cache);
+    for (int d = lane; d < a.hd; d += 64) {
+      const float val = d < a.vdim ? v[d] : 0.0f;
+      if constexpr (sizeof(T) == 2) gm_store(vc + (((size_t)page * a.kv_heads + h) * a.hd + d) * a.page_size + slot, val);   // [kv head][element][slot]
+      else gm_store(vc + (((size_t)page * a.kv_heads + h) * a.page_size + slot) * a.hd + d, val);
+    }
+    return;
+  }
+  const float* v = a.src + (size_t)row * a.lds + (size_t)hh * a.dim;
+  const int half = a.rot / 2, pairs = (a.dim + 1) / 2;
+  const float* ct = a.cos_table + (size_t)pos * half;
+  const float* st = a.sin_table + (size_t)pos * half;
+  // up to 256 elements a head: two pairs a lane
+  float e0[2], e1[2];
+  float acc = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int p = lane + 64 * j;
+    e0[j] = e1[j] = 0.0f;
+    if (p < pairs) {
+      const float x1 = v[2 * p], x2 = 2 * p + 1 < a.dim ? v[2 * p + 1] : 0.0f;
+      if (p < half) {
+        const float c = ct[p], s = st[p];
+        e0[j] = x1 * c - x2 * s;
+        e1[j] = x2 * c + x1 * s;
+      } else {
+        e0[j] = x1;
+        e1[j] = x2;
+      }
+      acc = fmaf(e0[j], e0[j], acc);
+      acc = fmaf(e1[j], e1[j], acc);
+    }
+  }
+  float inv = 1.0f;
+  if (a.unit_norm) {
+    acc = wave_sum(acc);
+    inv = 1.0f / sqrtf(acc / (float)a.dim + a.eps);
+  }
+  T* dst;
+  if (is_q) dst = reinterpret_cast<T*>(a.q_out) + (size_t)row * a.heads * a.hd + (size_t)hh * a.hd;
+  else dst = reinterpret_cast<T*>(a.k_cache) + (((size_t)page * a.kv_heads + (hh - a.heads)) * a.page_size + slot) * a.hd;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int p = lane + 64 * j;
+    if (2 * p < a.hd) gm_store(dst + 2 * p, 2 * p < a.dim ? e0[j] * inv : 0.0f);
+    if (2 * p + 1 < a.hd) gm_store(dst + 2 * p + 1, 2 * p + 1 < a.dim ? e1[j] * inv : 0.0f);
+  }
+}
+
+extern "C" int bw_pair_rope_unit(const float* src, int lds, const int32_t* positions, const int32_t* row_seq,
+                                 const int32_t* block_table, int table_stride, const float* cos_table, const float* sin_table,
+                                 void* q_out, void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads,
+                                 int dim, int vdim, int hd, int rot, int page_size, int unit_norm, float eps, int has_kv,
+                                 int write_cache, void* stream) {
+  if (rows <= 0) return 0;
+  if (dim > 256 || hd > 256 || dim > hd || vdim > hd || rot % 2 || rot > dim || page_size <= 0) return -2;
+  PairRopeArgs a{src, positions, row_seq, block_table, cos_table, sin_table, q_out, k_cache, v_cache, lds, rows, heads, kv_heads,
+                 dim, vdim, hd, rot, page_size, table_stride, unit_norm, has_kv, write_cache, eps};
+  const long long items = (long long)rows * (heads + (has_kv ? 2 * kv_heads : 0));
+  const dim3 grid((unsigned)((items + 3) / 4));
+  if (is_bf16) hipLaunchKernelGGL(pair_rope_unit_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(pair_rope_unit_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, a);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ output gate
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void gate_mul_kernel(const TI* __restrict__ av, int lda, int hd, const float* __restrict__ g, int ldg,
+                                                       TO* __restrict__ out, int ldo, int rows, int heads, int vdim) {
+  const int row = blockIdx.y;
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= heads * vdim) return;
+  const int h = e / vdim, d = e % vdim;
+  const float x = gm_load(av + (size_t)row * lda + (size_t)h * hd + d);
+  gm_store(out + (size_t)row * ldo + e, x * gm_sigmoid(g[(size_t)row * ldg + e]));
+}
+
+extern "C" int bw_gate_mul(const void* av, int a_is_bf16, int lda, int hd, const float* g, int ldg, void* out, int out_is_bf16,
+                           int ldo, int rows, int heads, int vdim, void* stream) {
+  if (rows <= 0) return 0;
+  if (rows > 65535 * 16) return -2;
+  const dim3 grid((heads * vdim + 255) / 256, rows);
+  hipStream_t s = (hipStream_t)stream;
+  if (a_is_bf16 && out_is_bf16)
+    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)av, lda, hd, g, ldg, (bf16_t*)out, ldo, rows, heads, vdim);
+  else if (a_is_bf16)
+    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, float>), grid, dim3(256), 0, s, (const bf16_t*)av, lda, hd, g, ldg, (float*)out, ldo, rows, heads, vdim);
+  else if (out_is_bf16)
+    hipLaunchKernelGGL((gate_mul_kernel<float, bf16_t>), grid, dim3(256), 0, s, (const float*)av, lda, hd, g, ldg, (bf16_t*)out, ldo, rows, heads, vdim);
+  else
+    hipLaunchKernelGGL((gate_mul_kernel<float, float>), grid, dim3(256), 0, s, (const float*)av, lda, hd, g, ldg, (float*)out, ldo, rows, heads, vdim);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ gated linear recurrence per channel
+
+struct RglruArgs {
+  const float* y;         // [rows, ldy]: the gate branch before its activation
+  const float* u;         // [rows, ldu]: the convolved recurrent branch
+  const float* gates;     // [rows, ldg]: per block of bs channels, bs recurrence-gate logits then bs input-gate logits
+  const float* ra_bias;   // [channels]
+  const float* ri_bias;
+  const float* decay;     // [channels]: c = -scale * softplus(lambda), so that log a = c * r
+  float* state;           // [slots, state_ld]: S [channels] at the pointer
+  void* out;              // [rows, ldo]
+  const int32_t* seq_rows;
+  const int32_t* slots;
+  const int32_t* positions;
+  long long state_ld;
+  int ldy, ldu, ldg, ldo, channels, bs;
+};
+
+__device__ __forceinline__ float gm_gelu_tanh(float z) {
+  const float inner = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  return 0.5f * z * (1.0f + tanhf(inner));
+}
+
+// What a token adds to its channel's state and the factor the state keeps: independent of the state itself.
+__device__ __forceinline__ void rglru_terms(float zr, float zi, float u, float br, float bi, float c, float& a, float& b) {
+  const float r = gm_sigmoid(zr + br), i = gm_sigmoid(zi + bi);
+  const float log_a = c * r;
+  a = bw_expf(log_a);
+  b = sqrtf(-expm1f(2.0f * log_a)) * (i * u);      // sqrt(1 - a^2) without the cancellation near a = 1
+}
+
+template <typename TO>
+__global__ __launch_bounds__(64) void rglru_scan_kernel(RglruArgs p) {
+  const int c = blockIdx.x * 64 + threadIdx.x, seq = blockIdx.y;
+  const int first = p.seq_rows[2 * seq], n = p.seq_rows[2 * seq + 1], slot = p.slots[seq];
+  if (c >= p.channels || n <= 0 || slot < 0 || p.positions[first] < 0) return;
+  const int blk = c / p.bs, o = c % p.bs;
+  const float br = p.ra_bias[c], bi = p.ri_bias[c], dc = p.decay[c];
+  const float* zr = p.gates + (size_t)first * p.ldg + (size_t)blk * 2 * p.bs + o;
+  const float* zi = zr + p.bs;
+  const float* u = p.u + (size_t)first * p.ldu + c;
+  const float* y = p.y + (size_t)first * p.ldy + c;
+  TO* out = reinterpret_cast<TO*>(p.out) + (size_t)first * p.ldo + c;
+  float* st = p.state + (size_t)slot * p.state_ld + c;
+  float S = *st;
+  constexpr int UN = 4;
+  int t = 0;
+  for (; t + UN <= n; t += UN) {
+    float vzr[UN], vzi[UN], vu[UN], vy[UN];
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      vzr[j] = zr[(size_t)(t + j) * p.ldg];
+      vzi[j] = zi[(size_t)(t + j) * p.ldg];
+      vu[j] = u[(size_t)(t + j) * p.ldu];
+      vy[j] = y[(size_t)(t + j) * p.ldy];
+    }
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      float a, b;
+      rglru_terms(vzr[j], vzi[j], vu[j], br, bi, dc, a, b);
+      S = fmaf(a, S, b);
+      gm_store(out + (size_t)(t + j) * p.ldo, S * gm_gelu_tanh(vy[j]));
+    }
+  }
+  for (; t < n; ++t) {
+    float a, b;
+    rglru_terms(zr[(size_t)t * p.ldg], zi[(size_t)t * p.ldg], u[(size_t)t * p.ldu], br, bi, dc, a, b);
+    S = fmaf(a, S, b);
+    gm_store(out + (size_t)t * p.ldo, S * gm_gelu_tanh(y[(size_t)t * p.ldy]));
+  }
+  *st = S;
+}
+
+extern "C" int bw_rglru_scan(const float* y, int ldy, const float* u, int ldu, const float* gates, int ldg, const float* ra_bias,
+                             const float* ri_bias, const float* decay, float* state, long long state_ld, void* out,
+                             int out_is_bf16, int ldo, const int32_t* seq_rows, const int32_t* slots, const int32_t* positions,
+                             int nseq, int channels, int bs, void* stream) {
+  if (nseq <= 0 || channels <= 0) return 0;
+  if (bs <= 0 || channels % bs || nseq > 65535) return -2;
+  RglruArgs p{y, u, gates, ra_bias, ri_bias, decay, state, out, seq_rows, slots, positions, state_ld, ldy, ldu, ldg, ldo, channels, bs};
+  const dim3 grid((channels + 63) / 64, nseq);
+  if (out_is_bf16) hipLaunchKernelGGL(rglru_scan_kernel<bf16_t>, grid, dim3(64), 0, (hipStream_t)stream, p);
+  else hipLaunchKernelGGL(rglru_scan_kernel<float>, grid, dim3(64), 0, (hipStream_t)stream, p);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ x += rmsnorm(y) * w
+
+template <typename WT>
+__global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__ y, int ldy, const WT* __restrict__ w, float* __restrict__ x,
+                                                       int ldx, int rows, int dim, float eps) {
+  const int row = blockIdx.x * 4 + wave_index(), lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const float* yr = y + (size_t)row * ldy;
+  float acc = 0.0f;
+  for (int e = lane; e < dim; e += 64) acc = fmaf(yr[e], yr[e], acc);
+  acc = wave_sum(acc);
+  const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
+  float* xr = x + (size_t)row * ldx;
+  for (int e = lane; e < dim; e += 64) xr[e] = xr[e] + (yr[e] * inv) * gm_load(w + e);
+}
+
+extern "C" int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, int rows, int dim, float eps,
+                           void* stream) {
+  if (rows <= 0) return 0;
+  const dim3 grid((rows + 3) / 4);
+  if (w_is_bf16) hipLaunchKernelGGL(norm_add_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const bf16_t*)w, x, ldx, rows, dim, eps);
+  else hipLaunchKernelGGL(norm_add_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const float*)w, x, ldx, rows, dim, eps);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ soft cap
+
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, int ld, int cols, float cap) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= cols) return;
+  float* p = x + (size_t)blockIdx.y * ld + e;
+  *p = cap * tanhf(*p / cap);
+}
+
+extern "C" int bw_softcap(float* x, int ld, int rows, int cols, float cap, void* stream) {
+  if (rows <= 0 || cols <= 0) return 0;
+  if (!(cap > 0.0f) || rows > 65535) return -2;
+  hipLaunchKernelGGL(softcap_kernel, dim3((cols + 255) / 256, rows), dim3(256), 0, (hipStream_t)stream, x, ld, cols, cap);
+  return BW_LAUNCH_CHECK();
+}

@@ -1,0 +1,377 @@
+// A feed-forward of routed experts.
+//
+//   route:    per row, scores = softmax of the router's logits over all experts; experts lie in equal groups of
+//             neighbours, a group's score is its best expert's, only experts of the `keep` best groups can be chosen;
+//             the `top` best of those are the row's experts, weighted by their scores as they are.  Ties go to the
+//             lower index.  All 32-bit.
+//   plan:     the step's (row, choice) pairs ("slots") sorted by expert into runs, and the runs cut into tiles of
+//             MOE_TM slots: every tile belongs to one expert.  Built on the device; the products' grids are sized for
+//             the worst case and tiles past the last return at once.
+//   gate_up:  per tile, G = X W_gate^T and U = X W_up^T of its expert, then h = min(G, limit) * sigmoid(alpha * min(G, limit))
+//             * (clamp(U, -limit, limit) + 1), stored by the slot's place in the sorted order
+//   down:     per tile, h W_down^T of its expert, 32-bit sums by sorted place
+//   combine:  out[row] = sum over the row's choices, in the order they were chosen, of weight * its expert's output
+//
+// bfloat16 mode runs the two products on the matrix cores (v_mfma_f32_16x16x32_bf16 over the inner size ascending from
+// zero, one accumulator per 16 x 16 block of outputs): what a row gets depends on the row and its expert alone, not on
+// the rows it shares a tile with.  The 32-bit mode runs one fused multiply-add chain per output over the inner size
+// ascending.
+#include <math.h>
+
+#include "common.h"
+#include "api.h"
+
+#define MOE_TM 32            // slots a tile
+#define MOE_MAX_EXPERTS 1024
+
+// ------------------------------------------------------------------------------ route
+
+// (value, index) of the wave's best: larger value first, then lower index
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(v, off, 64);
+    const int oi = __shfl_xor(i, off, 64);
+    const bool take = ov > v || (ov == v && oi < i);
+    v = take ? ov : v;
+    i = take ? oi : i;
+  }
+}
+
+// A wave a row.  LDS per wave: scores [E], group scores [count], allowed [count].
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, int rows, int E, int top, int count,
+                                                        int keep, int32_t* __restrict__ ids, float* __restrict__ wts) {
+  extern __shared__ float route_lds[];
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  float* s = route_lds + (size_t)wave * (E + 2 * count);
+  float* gs = s + E;
+  float* allowed = gs + count;
+  const float* z = logits + (size_t)row * ld;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+  mx = wave_max(mx);
+  float sum = 0.0f;
+  for (int e = lane; e < E; e += 64) {
+    const float ex = bw_expf(z[e] - mx);
+    s[e] = ex;
+    sum += ex;
+  }
+  sum = wave_sum(sum);
+  for (int e = lane; e < E; e += 64) s[e] = s[e] / sum;
+  __builtin_amdgcn_wave_barrier();
+  const int gsz = E / count;
+  for (int g = lane; g < count; g += 64) {
+    float best = -1.0f;
+    for (int j = 0; j < gsz; ++j) best = fmaxf(best, s[g * gsz + j]);
+    gs[g] = best;
+    allowed[g] = keep >= count ? 1.0f : 0.0f;
+  }
+  __builtin_amdgcn_wave_barrier();
+  if (keep < count) {
+    for (int it = 0; it < keep; ++it) {
+      float v = -2.0f;
+      int i = 0x7fffffff;
+      for (int g = lane; g < count; g += 64)
+        if (gs[g] > v) { v = gs[g]; i = g; }
+      wave_argmax(v, i);
+      if (lane == 0) { gs[i] = -3.0f; allowed[i] = 1.0f; }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+  for (int it = 0; it < top; ++it) {
+    float v = -2.0f;
+    int i = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float sc = allowed[e / gsz] > 0.0f ? s[e] : -2.0f;
+      if (sc > v) { v = sc; i = e; }
+    }
+    wave_argmax(v, i);
+    if (lane == 0) {
+      ids[(size_t)row * top + it] = i;
+      wts[(size_t)row * top + it] = v;
+      s[i] = -3.0f;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+extern "C" int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
+                            float* wts, void* stream) {
+  if (rows <= 0) return 0;
+  if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || groups < 1 || experts % groups || keep < 1 || keep > groups ||
+      top > keep * (experts / groups))
+    return -2;
+  const size_t bytes = (size_t)4 * (experts + 2 * groups) * sizeof(float);
+  hipLaunchKernelGGL(moe_route_kernel, dim3((rows + 3) / 4), dim3(256), bytes, (hipStream_t)stream, logits, ld, rows, experts, top,
+                     groups, keep, ids, wts);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ plan
+
+// One workgroup.  sorted[p] = slot at sorted place p; place[slot] = p; tiles[t] = (expert, first place, slots, 0);
+// meta[0] = number of tiles.  Within an expert's run the slots ascend (every thread ranks its slots by counting the
+// equal experts before them), so the plan is the same from run to run.
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ ids, int n, int E, int32_t* __restrict__ sorted,
+                                                        int32_t* __restrict__ place, int32_t* __restrict__ tiles,
+                                                        int32_t* __restrict__ meta, int32_t* __restrict__ rank) {
+  __shared__ int counts[MOE_MAX_EXPERTS], start[MOE_MAX_EXPERTS], tile0[MOE_MAX_EXPERTS];
+  __shared__ int chunk_counts[MOE_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += 1024) counts[e] = 0;
+  __syncthreads();
+  // the rank of a slot among the slots of its expert, in slot order: chunks of 1024 slots, one after the other
+  for (int base = 0; base < n; base += 1024) {
+    for (int e = tid; e < E; e += 1024) chunk_counts[e] = 0;
+    __syncthreads();
+    const int sidx = base + tid;
+    int e = -1;
+    if (sidx < n) e = ids[sidx];
+    // rank inside the chunk: ballot per wave would do; with few experts a count over the chunk's earlier slots through
+    // LDS atomics gives an order that changes from run to run, so the earlier slots are counted directly
+    __shared__ int chunk_ids[1024];
+    chunk_ids[tid] = e;
+    __syncthreads();
+    if (e >= 0) {
+      int before = 0;
+      for (int j = 0; j < tid; ++j) before += chunk_ids[j] == e;
+      rank[sidx] = counts[e] + before;
+      atomicAdd(&chunk_counts[e], 1);
+    }
+    __syncthreads();
+    for (int x = tid; x < E; x += 1024) counts[x] += chunk_counts[x];
+    __syncthreads();
+  }
+  if (tid == 0) {
+    int s0 = 0, t0 = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = s0;
+      tile0[e] = t0;
+      s0 += counts[e];
+      t0 += (counts[e] + MOE_TM - 1) / MOE_TM;
+    }
+    meta[0] = t0;
+  }
+  __syncthreads();
+  for (int sidx = tid; sidx < n; sidx += 1024) {
+    const int e = ids[sidx];
+    const int p = start[e] + rank[sidx];
+    sorted[p] = sidx;
+    place[sidx] = p;
+  }
+  for (int e = tid; e < E; e += 1024) {
+    const int nt = (counts[e] + MOE_TM - 1) / MOE_TM;
+    for (int t = 0; t < nt; ++t) {
+      int32_t* rec = tiles + (size_t)(tile0[e] + t) * 4;
+      rec[0] = e;
+      rec[1] = start[e] + t * MOE_TM;
+      rec[2] = min(MOE_TM, counts[e] - t * MOE_TM);
+      rec[3] = 0;
+    }
+  }
+}
+
+extern "C" int bw_moe_max_tiles(int slots, int experts) {
+  const int full = slots / MOE_TM;
+  return full + (experts < slots ? experts : slots);
+}
+
+extern "C" int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* sorted, int32_t* place, int32_t* tiles,
+                           int32_t* meta, int32_t* rank, void* stream) {
+  if (slots <= 0) return 0;
+  if (experts < 1 || experts > MOE_MAX_EXPERTS) return -2;
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ids, slots, experts, sorted, place, tiles, meta, rank);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ the experts' activation
+
+__device__ __forceinline__ float moe_act(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return (g * (1.0f / (1.0f + bw_expf(-alpha * g)))) * (u + 1.0f);
+}
+
+// ------------------------------------------------------------------------------ products on the matrix cores
+
+struct MoeArgs {
+  const int32_t* sorted;   // [slots]
+  const int32_t* tiles;    // [max_tiles][4]
+  const int32_t* meta;
+  int top, K, N;           // inner size, output columns of the product (ff for gate_up, width for down)
+  float limit, alpha;
+};
+
+// A workgroup of four waves per (tile of MOE_TM slots, 128 output columns); a wave owns 32 columns, for GATE_UP of
+// the gate and of the up matrix both.  Operands go from memory straight into registers: lane (r, g) holds row r's
+// (or column r's) elements k + 8g .. k + 8g + 7.  Rows of a tile past its slots read row 0 of x and are never stored.
+template <bool GATE_UP>
+__global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w,
+                                                       void* __restrict__ out, int ldo) {
+  const int tile = blockIdx.y;
+  if (tile >= a.meta[0]) return;
+  const int wave = wave_index(), lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int e = a.tiles[tile * 4], p0 = a.tiles[tile * 4 + 1], cnt = a.tiles[tile * 4 + 2];
+  const int n0 = blockIdx.x * 128 + wave * 32;
+  if (n0 >= a.N) return;                                   // (scalar: the wave's columns lie past the matrix)
+  constexpr int NB = GATE_UP ? 4 : 2, MB = MOE_TM / 16;
+  const bf16_t* xr[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int q = 16 * i + r;
+    size_t src_row = 0;
+    if (q < cnt) src_row = GATE_UP ? (size_t)(a.sorted[p0 + q] / a.top) : (size_t)(p0 + q);
+    else if (!GATE_UP) src_row = (size_t)p0;
+    else src_row = (size_t)(a.sorted[p0] / a.top);
+    xr[i] = x + src_row * ldx + 8 * g;
+  }
+  // weights of expert e: GATE_UP [2N, K] (gate rows, then up rows), else [N, K]
+  const bf16_t* wr[NB];
+  const size_t wbase = (size_t)e * (GATE_UP ? 2 : 1) * a.N * a.K;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int half = GATE_UP ? b >> 1 : 0, cb = GATE_UP ? b & 1 : b;
+    const int n = min(n0 + 16 * cb + r, a.N - 1);
+    wr[b] = w + wbase + ((size_t)half * a.N + n) * a.K + 8 * g;
+  }
+  f32x4 acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  const int K = a.K;
+  auto load = [&](int k, u32x4 (&af)[MB], u32x4 (&bfr)[NB]) {
+    const bool live = k + 8 * g + 8 <= K;                  // (K is a multiple of 8)
+#pragma unroll
+    for (int i = 0; i < MB; ++i) af[i] = live ? *reinterpret_cast<const u32x4*>(xr[i] + k) : zero;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) bfr[b] = live ? *reinterpret_cast<const u32x4*>(wr[b] + k) : zero;
+  };
+  u32x4 a0[MB], b0[NB], a1[MB], b1[NB];
+  load(0, a0, b0);
+  for (int k = 0; k < K; k += 64) {
+    if (k + 32 < K) load(k + 32, a1, b1);
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a0[i]), as_bf16x8(b0[b]), acc[i][b], 0, 0, 0);
+    if (k + 32 < K) {                                       // (scalar)
+      if (k + 64 < K) load(k + 64, a0, b0);
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+          acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a1[i]), as_bf16x8(b1[b]), acc[i][b], 0, 0, 0);
+    }
+  }
+  // accumulator element q of block (i, b): slot 16 i + 4 g + q, column 16 b' + r
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = 16 * i + 4 * g + q;
+      if (m >= cnt) continue;
+      if constexpr (GATE_UP) {
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+          const int n = n0 + 16 * cb + r;
+          if (n < a.N)
+            reinterpret_cast<bf16_t*>(out)[(size_t)(p0 + m) * ldo + n] = f32_to_bf16(moe_act(acc[i][cb][q], acc[i][2 + cb][q], a.limit, a.alpha));
+        }
+      } else {
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+          const int n = n0 + 16 * cb + r;
+          if (n < a.N) reinterpret_cast<float*>(out)[(size_t)(p0 + m) * ldo + n] = acc[i][cb][q];
+        }
+      }
+    }
+}
+
+// ------------------------------------------------------------------------------ products in 32-bit
+
+// A thread an output (sorted place, column): one chain of fused multiply-adds over the inner size ascending.
+// ROUND: the activation is rounded to bfloat16 (and kept as a 32-bit value), for the bfloat16 mode of weights that the
+// matrix-core kernels do not take.
+template <bool GATE_UP, typename WT>
+__global__ __launch_bounds__(64) void moe_f32_kernel(MoeArgs a, const float* __restrict__ x, int ldx, const WT* __restrict__ w,
+                                                     float* __restrict__ out, int ldo, int round_out) {
+  const int tile = blockIdx.y;
+  if (tile >= a.meta[0]) return;
+  const int e = a.tiles[tile * 4], p0 = a.tiles[tile * 4 + 1], cnt = a.tiles[tile * 4 + 2];
+  const int n = blockIdx.x * 64 + threadIdx.x;
+  if (n >= a.N) return;
+  const size_t wbase = (size_t)e * (GATE_UP ? 2 : 1) * a.N * a.K;
+  const WT* wg = w + wbase + (size_t)n * a.K;
+  const WT* wu = wg + (size_t)a.N * a.K;
+  for (int m = 0; m < cnt; ++m) {
+    const float* xr = x + (GATE_UP ? (size_t)(a.sorted[p0 + m] / a.top) : (size_t)(p0 + m)) * ldx;
+    float sg = 0.0f, su = 0.0f;
+    for (int k = 0; k < a.K; ++k) {
+      const float xv = xr[k];
+      if constexpr (sizeof(WT) == 2) {
+        sg = fmaf(xv, bf16_to_f32(wg[k]), sg);
+        if (GATE_UP) su = fmaf(xv, bf16_to_f32(wu[k]), su);
+      } else {
+        sg = fmaf(xv, wg[k], sg);
+        if (GATE_UP) su = fmaf(xv, wu[k], su);
+      }
+    }
+    float y = GATE_UP ? moe_act(sg, su, a.limit, a.alpha) : sg;
+    if (GATE_UP && round_out) y = bf16_to_f32(f32_to_bf16(y));
+    out[(size_t)(p0 + m) * ldo + n] = y;
+  }
+}
+
+extern "C" int bw_moe_experts(const void* x, int x_is_bf16, int ldx, const void* w, int w_is_bf16, void* out, int ldo,
+                              const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int max_tiles, int top, int K,
+                              int N, int gate_up, float limit, float alpha, int round_out, void* stream) {
+  if (max_tiles <= 0) return 0;
+  if (max_tiles > 65535 || K <= 0 || N <= 0) return -2;
+  MoeArgs a{sorted, tiles, meta, top, K, N, limit, alpha};
+  hipStream_t s = (hipStream_t)stream;
+  if (x_is_bf16) {
+    if (!w_is_bf16 || K % 8 || ldx % 8) return -3;
+    const dim3 grid((N + 127) / 128, max_tiles);
+    if (gate_up) hipLaunchKernelGGL(moe_mfma_kernel<true>, grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+    else hipLaunchKernelGGL(moe_mfma_kernel<false>, grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+    return BW_LAUNCH_CHECK();
+  }
+  const dim3 grid((N + 63) / 64, max_tiles);
+  if (gate_up) {
+    if (w_is_bf16) hipLaunchKernelGGL((moe_f32_kernel<true, bf16_t>), grid, dim3(64), 0, s, a, (const float*)x, ldx, (const bf16_t*)w, (float*)out, ldo, round_out);
+    else hipLaunchKernelGGL((moe_f32_kernel<true, float>), grid, dim3(64), 0, s, a, (const float*)x, ldx, (const float*)w, (float*)out, ldo, round_out);
+  } else {
+    if (w_is_bf16) hipLaunchKernelGGL((moe_f32_kernel<false, bf16_t>), grid, dim3(64), 0, s, a, (const float*)x, ldx, (const bf16_t*)w, (float*)out, ldo, 0);
+    else hipLaunchKernelGGL((moe_f32_kernel<false, float>), grid, dim3(64), 0, s, a, (const float*)x, ldx, (const float*)w, (float*)out, ldo, 0);
+  }
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ combine
+
+// out[row][c] (=, or +=) sum_j wts[row][j] * y[place[row * top + j]][c], j ascending, one chain per element.
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, int ldy, const int32_t* __restrict__ place,
+                                                          const float* __restrict__ wts, int top, float* __restrict__ out, int ldo,
+                                                          int width, int accumulate) {
+  const int row = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  float acc = 0.0f;
+  for (int j = 0; j < top; ++j)
+    acc = fmaf(wts[(size_t)row * top + j], y[(size_t)place[(size_t)row * top + j] * ldy + c], acc);
+  float* o = out + (size_t)row * ldo + c;
+  *o = accumulate ? *o + acc : acc;
+}
+
+extern "C" int bw_moe_combine(const float* y, int ldy, const int32_t* place, const float* wts, int top, float* out, int ldo,
+                              int rows, int width, int accumulate, void* stream) {
+  if (rows <= 0) return 0;
+  if (rows > 65535) return -2;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((width + 255) / 256, rows), dim3(256), 0, (hipStream_t)stream, y, ldy, place, wts, top,
+                     out, ldo, width, accumulate);
+  return BW_LAUNCH_CHECK();
+}

@@ -55,12 +55,12 @@ _SIGS = {
     "bw_gemm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_attention_f32_tiles": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p,
-                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p],
     "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p],
     "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_longlong,
-                          c_void_p, c_int, c_void_p],
+                          c_void_p, c_int, c_void_p, c_void_p],
     "bw_attention_decode_scratch": [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     "bw_attention_fold_group_tiles": [c_int],
     "bw_norm_gemm_supported": [c_int, c_int],
@@ -92,6 +92,22 @@ _SIGS = {
                        c_void_p],
     "bw_headwise_linear": [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
                            c_int, c_void_p],
+    "bw_causal_conv": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_longlong, c_void_p, c_void_p,
+                       c_void_p, c_int, c_int, c_void_p, c_int, c_void_p],
+    "bw_pair_rope_unit": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                          c_int, c_void_p],
+    "bw_gate_mul": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_rglru_scan": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
+                      c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "bw_norm_add": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+    "bw_softcap": [c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+    "bw_moe_route": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "bw_moe_max_tiles": [c_int, c_int],
+    "bw_moe_plan": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "bw_moe_experts": [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                       c_int, c_int, c_int, c_float, c_float, c_int, c_void_p],
+    "bw_moe_combine": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "bw_shared_key_attention": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int,
                                 c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
 }
@@ -105,7 +121,7 @@ _fns = {}
 _CHAIN_KEEPS = frozenset({
     "bw_gemm_bf16", "bw_gemm_add_bf16", "bw_norm_gemm_bf16", "bw_norm_qkv_rope_bf16",
     "bw_gemm_add_scratch", "bw_norm_gemm_supported", "bw_norm_gemm_wide_supported", "bw_attention_decode_scratch",
-    "bw_attention_fold_group_tiles", "bw_gemm_add_bf16_static_max", "bw_chain_sync_words", "bw_chain_begin",
+    "bw_attention_fold_group_tiles", "bw_gemm_add_bf16_static_max", "bw_moe_max_tiles", "bw_chain_sync_words", "bw_chain_begin",
     "bw_chain_flush", "bw_chain_end",
 })
 _chain_open = False
@@ -485,9 +501,21 @@ def norm_qkv_rope_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w
 
 # ------------------------------------------------------------------------------ attention
 
+def _sink_ptr(sink: Optional[torch.Tensor], heads: int) -> int:
+    """``sink`` [heads] float32: a score per head that joins the softmax's denominator as exp(sink) and has no value
+    (the score scale does not apply to it); None: no sink."""
+    if sink is None:
+        return 0
+    _need(sink, torch.float32, "sink")
+    if sink.numel() != heads:
+        raise ValueError("attention: a sink per head is needed")
+    return sink.data_ptr()
+
+
 def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
                   k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, rows: int, heads: int,
-                  kv_heads: int, head_dim: int, page_size: int, window: int, scale: float) -> None:
+                  kv_heads: int, head_dim: int, page_size: int, window: int, scale: float,
+                  sink: Optional[torch.Tensor] = None) -> None:
     """q: [rows, stride] float32 with head h at columns h*head_dim.. (the stacked q|k|v rows
     serve as they are); caches [pages, kv_heads, page_size, head_dim] float32."""
     _need(q, torch.float32, "q")
@@ -506,12 +534,13 @@ def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tenso
     _check(_fn("bw_attention_f32")(q.data_ptr(), q.stride(0), positions.data_ptr(), row_seq.data_ptr(),
                                    block_table.data_ptr(), block_table.stride(0), k_cache.data_ptr(),
                                    v_cache.data_ptr(), out.data_ptr(), out.stride(0), rows, heads, kv_heads, head_dim,
-                                   page_size, int(window), float(scale), _stream()), "attention_f32")
+                                   page_size, int(window), float(scale), _sink_ptr(sink, heads), _stream()), "attention_f32")
 
 
 def attention_f32_tiles(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor,
                         num_tiles: int, tiled, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
-                        heads: int, kv_heads: int, head_dim: int, page_size: int, window: int, scale: float) -> None:
+                        heads: int, kv_heads: int, head_dim: int, page_size: int, window: int, scale: float,
+                        sink: Optional[torch.Tensor] = None) -> None:
     """``attention_f32`` over tiles ([tiles, 4] int32 = first row, rows, request, 0; a tile's rows are consecutive
     rows of one request).  ``tiled`` True (1): a workgroup per tile of up to 16 rows, keys and values shared
     through LDS; 2: a wave per tile of up to 32 rows, both products as chains of single-step matrix instructions
@@ -533,7 +562,8 @@ def attention_f32_tiles(q: torch.Tensor, positions: torch.Tensor, block_table: t
     _check(_fn("bw_attention_f32_tiles")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
                                          block_table.stride(0), tiles.data_ptr(), int(num_tiles), int(tiled),
                                          k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads,
-                                         kv_heads, head_dim, page_size, int(window), float(scale), _stream()),
+                                         kv_heads, head_dim, page_size, int(window), float(scale), _sink_ptr(sink, heads),
+                                         _stream()),
            "attention_f32_tiles")
 
 
@@ -541,7 +571,7 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
                    tiles: Optional[torch.Tensor], num_tiles: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                    out: torch.Tensor, heads: int, kv_heads: int, head_dim: int, page_size: int, window: int,
                    scale: float, decode: bool = False,
-                   scratch: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> None:
+                   scratch: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, sink: Optional[torch.Tensor] = None) -> None:
     """q, out: [rows, heads*head_dim] bfloat16; k pages [kv_heads, page, hd], v pages
     [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0).
 
@@ -590,7 +620,7 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
                                     out.stride(0), heads, kv_heads, head_dim, page_size, int(window), float(scale), int(decode),
                                     sc_f.data_ptr() if sc_f is not None else 0, sc_f.numel() if sc_f is not None else 0,
                                     sc_c.data_ptr() if sc_c is not None else 0, sc_c.numel() if sc_c is not None else 0,
-                                    _stream()),
+                                    _sink_ptr(sink, heads), _stream()),
            "attention_bf16")
 
 
@@ -908,6 +938,216 @@ def shared_key_attention_mfma(q: torch.Tensor, positions: torch.Tensor, block_ta
                                                int(kchunk), 0 if partial is None else partial.data_ptr(),
                                                0 if partial is None else partial.numel(), _stream()),
            "shared_key_attention_mfma")
+
+
+# ------------------------------------------------------------------------------ convolved, gated and recurrent mixers
+
+CONV_MAX_TAPS = 8
+
+
+def causal_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
+                seq_rows: torch.Tensor, slots: torch.Tensor, positions: torch.Tensor, nseq: int, max_seq_rows: int,
+                out: torch.Tensor) -> None:
+    """out[t, c] = sum_j weight[c, j] * x[t - taps + 1 + j, c] (+ bias[c]) along every request's rows, the inputs before a
+    portion's first row taken from ``state`` [slots, >= (taps - 1) * channels] (a view may start inside a wider slot),
+    which then receives the portion's last taps - 1 inputs.  ``x`` [rows, >= channels] float32 (rows apart by its
+    stride), ``out`` likewise.  ``max_seq_rows``: the most rows a request brings in this step."""
+    if x.dtype != torch.float32 or out.dtype != torch.float32 or x.stride(1) != 1 or out.stride(1) != 1 or not (x.is_cuda and out.is_cuda):
+        raise ValueError("causal_conv: x and out must be float32 GPU matrices with contiguous rows")
+    if weight.dim() != 2 or not weight.is_cuda or not weight.is_contiguous():
+        raise ValueError("causal_conv: weight must be a contiguous [channels, taps] GPU tensor")
+    channels, taps = weight.shape
+    wb = _is_bf16(weight, "weight")
+    if taps < 1 or taps > CONV_MAX_TAPS:
+        raise ValueError(f"causal_conv: {taps} taps; the kernel takes 1 to {CONV_MAX_TAPS}")
+    if x.shape[1] < channels or out.shape[1] < channels:
+        raise ValueError("causal_conv: x or out narrower than the channels")
+    if bias is not None and (bias.dtype != weight.dtype or bias.numel() != channels or not bias.is_contiguous()):
+        raise ValueError("causal_conv: bias must be [channels] of the weight's dtype")
+    for t, what in ((seq_rows, "seq_rows"), (slots, "slots"), (positions, "positions")):
+        _need(t, torch.int32, what)
+    if seq_rows.numel() < 2 * nseq or slots.numel() < nseq:
+        raise ValueError("causal_conv: fewer request records than requests")
+    sp, sld = 0, 0
+    if taps > 1:
+        if state is None or state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < (taps - 1) * channels:
+            raise ValueError(f"causal_conv: a state slot needs {(taps - 1) * channels} float32 elements")
+        sp, sld = state.data_ptr(), state.stride(0)
+    _check(_fn("bw_causal_conv")(x.data_ptr(), x.stride(0), weight.data_ptr(), 0 if bias is None else bias.data_ptr(), wb, taps,
+                                 channels, sp, sld, seq_rows.data_ptr(), slots.data_ptr(), positions.data_ptr(), int(nseq),
+                                 int(max_seq_rows), out.data_ptr(), out.stride(0), _stream()), "causal_conv")
+
+
+def pair_rope_unit(src: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
+                   cos: torch.Tensor, sin: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
+                   v_cache: Optional[torch.Tensor], rows: int, heads: int, kv_heads: int, dim: int, vdim: int, head_size: int,
+                   rot: int, page_size: int, unit_norm: bool, eps: float, has_kv: bool, write_cache: bool) -> None:
+    """``src`` [rows, >= heads*dim (+ kv_heads*(dim+vdim))] float32: query heads, then key heads, then value heads.  The
+    first ``rot`` elements of every query and key head are rotated pair by pair ((2i, 2i+1) by the angle of table
+    column i at the row's position), the head is then divided by its root mean square if ``unit_norm``; queries go to
+    ``q_out`` [rows, heads*head_size], keys and values (as they are) into the row's page slot, all padded with zeros
+    to ``head_size``.  Page layouts: bfloat16 keys [kv head][slot][element], values [kv head][element][slot]; float32
+    both [kv head][slot][element]."""
+    if src.dtype != torch.float32 or src.stride(1) != 1 or not src.is_cuda:
+        raise ValueError("pair_rope_unit: src must be a float32 GPU matrix with contiguous rows")
+    for t, what in ((positions, "positions"), (row_seq, "row_seq"), (block_table, "block_table")):
+        _need(t, torch.int32, what)
+    _need(cos, torch.float32, "cos table")
+    _need(sin, torch.float32, "sin table")
+    bf = _act_out(q_out, "q_out")
+    need = heads * dim + (kv_heads * (dim + vdim) if has_kv else 0)
+    if src.shape[1] < need or src.shape[0] < rows or q_out.shape[0] < rows or q_out.shape[1] != heads * head_size:
+        raise ValueError("pair_rope_unit: src or q_out do not fit")
+    if positions.numel() < rows or row_seq.numel() < rows:
+        raise ValueError("pair_rope_unit: fewer positions than rows")
+    if rot % 2 or rot > dim or (rot and (cos.shape[1] != rot // 2 or sin.shape != cos.shape)):
+        raise ValueError("pair_rope_unit: rotary tables must be [positions, rot/2]")
+    if max(dim, vdim) > head_size or head_size > 256:
+        raise ValueError("pair_rope_unit: heads of up to 256 elements, no larger than the cache's head size")
+    kp = vp = 0
+    if has_kv and write_cache:
+        page_elems = kv_heads * page_size * head_size
+        for c in (k_cache, v_cache):
+            if c is None or c.dtype != q_out.dtype or c.dim() != 2 or c.shape[1] != page_elems or not c.is_contiguous():
+                raise ValueError(f"pair_rope_unit: caches must be [pages, {page_elems}] of q_out's dtype")
+        kp, vp = k_cache.data_ptr(), v_cache.data_ptr()
+    _check(_fn("bw_pair_rope_unit")(src.data_ptr(), src.stride(0), positions.data_ptr(), row_seq.data_ptr(), block_table.data_ptr(),
+                                    block_table.stride(0), cos.data_ptr(), sin.data_ptr(), q_out.data_ptr(), kp, vp, bf, rows,
+                                    heads, kv_heads, dim, vdim, head_size, rot, page_size, int(unit_norm), float(eps),
+                                    int(has_kv), int(write_cache and has_kv), _stream()), "pair_rope_unit")
+
+
+def gate_mul(av: torch.Tensor, head_size: int, g: torch.Tensor, out: torch.Tensor, rows: int, heads: int, vdim: int) -> None:
+    """out[r, h*vdim + d] = av[r, h*head_size + d] * sigmoid(g[r, h*vdim + d]); ``g`` float32 (a column slice will do)."""
+    if g.dtype != torch.float32 or g.stride(1) != 1 or g.shape[1] < heads * vdim:
+        raise ValueError("gate_mul: g must be float32 with contiguous rows of heads*vdim")
+    if av.shape[1] != heads * head_size or out.shape[1] != heads * vdim or vdim > head_size:
+        raise ValueError("gate_mul: av or out do not fit")
+    if min(av.shape[0], out.shape[0], g.shape[0]) < rows:
+        raise ValueError("gate_mul: buffers shorter than the rows")
+    _check(_fn("bw_gate_mul")(av.data_ptr(), _act_out(av, "av"), av.stride(0), head_size, g.data_ptr(), g.stride(0), out.data_ptr(),
+                              _act_out(out, "out"), out.stride(0), rows, heads, vdim, _stream()), "gate_mul")
+
+
+def rglru_scan(y: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, ra_bias: torch.Tensor, ri_bias: torch.Tensor,
+               decay: torch.Tensor, state: torch.Tensor, out: torch.Tensor, seq_rows: torch.Tensor, slots: torch.Tensor,
+               positions: torch.Tensor, nseq: int, channels: int, block: int) -> None:
+    """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) * i_t * u_t per channel along every request's rows, from and to ``state``
+    [slots, >= channels]; a_t = exp(decay * r_t), r_t = sigmoid(gate logits + ra_bias), i_t likewise with ri_bias;
+    ``gates`` [rows, channels/block * 2*block]: per block its recurrence-gate logits, then its input-gate logits;
+    out = S_t * gelu_tanh(y_t).  y, u: float32 with contiguous rows (column slices will do)."""
+    for t, what in ((y, "y"), (u, "u"), (gates, "gates"), (state, "state")):
+        if t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or not t.is_cuda:
+            raise ValueError(f"rglru_scan: {what} must be a float32 GPU matrix with contiguous rows")
+    for t, what in ((ra_bias, "ra_bias"), (ri_bias, "ri_bias"), (decay, "decay")):
+        _need(t, torch.float32, what)
+        if t.numel() != channels:
+            raise ValueError(f"rglru_scan: {what} needs an element per channel")
+    for t, what in ((seq_rows, "seq_rows"), (slots, "slots"), (positions, "positions")):
+        _need(t, torch.int32, what)
+    if channels % block or min(y.shape[1], u.shape[1], state.shape[1]) < channels or gates.shape[1] < 2 * channels or out.shape[1] != channels:
+        raise ValueError("rglru_scan: widths do not fit the channels")
+    if seq_rows.numel() < 2 * nseq or slots.numel() < nseq:
+        raise ValueError("rglru_scan: fewer request records than requests")
+    _check(_fn("bw_rglru_scan")(y.data_ptr(), y.stride(0), u.data_ptr(), u.stride(0), gates.data_ptr(), gates.stride(0),
+                                ra_bias.data_ptr(), ri_bias.data_ptr(), decay.data_ptr(), state.data_ptr(), state.stride(0),
+                                out.data_ptr(), _act_out(out, "out"), out.stride(0), seq_rows.data_ptr(), slots.data_ptr(),
+                                positions.data_ptr(), int(nseq), channels, block, _stream()), "rglru_scan")
+
+
+def norm_add(y: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, rows: int, eps: float) -> None:
+    """x[:rows] += y / sqrt(mean(y^2) + eps) * weight, all 32-bit."""
+    _need(y, torch.float32, "y")
+    _need(x, torch.float32, "x")
+    dim = x.shape[1]
+    if y.shape[1] != dim or weight.numel() != dim or not weight.is_cuda or min(x.shape[0], y.shape[0]) < rows:
+        raise ValueError("norm_add: y, weight and x do not fit")
+    _check(_fn("bw_norm_add")(y.data_ptr(), y.stride(0), weight.data_ptr(), _is_bf16(weight, "weight"), x.data_ptr(), x.stride(0),
+                              rows, dim, float(eps), _stream()), "norm_add")
+
+
+def softcap(x: torch.Tensor, rows: int, cap: float) -> None:
+    """x[:rows] = cap * tanh(x / cap) in place."""
+    _need(x, torch.float32, "x")
+    if x.shape[0] < rows or not cap > 0:
+        raise ValueError("softcap: fewer rows than said, or a cap that is not positive")
+    _check(_fn("bw_softcap")(x.data_ptr(), x.stride(0), rows, x.shape[1], float(cap), _stream()), "softcap")
+
+
+# ------------------------------------------------------------------------------ routed experts
+
+def moe_max_tiles(slots: int, experts: int) -> int:
+    """The most tiles a plan of this many (row, choice) pairs over this many experts can have."""
+    return int(_fn("bw_moe_max_tiles")(int(slots), int(experts)))
+
+
+def moe_route(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int, ids: torch.Tensor, wts: torch.Tensor) -> None:
+    """Per row: softmax over the experts' logits; the ``top`` best experts among those of the ``keep`` best of ``groups``
+    equal groups of neighbours (a group's score: its best expert's); ``ids`` [rows, top] int32 in the order chosen,
+    ``wts`` [rows, top] their scores."""
+    _need(logits, torch.float32, "logits")
+    _need(ids, torch.int32, "ids")
+    _need(wts, torch.float32, "wts")
+    experts = logits.shape[1]
+    if logits.shape[0] < rows or ids.numel() < rows * top or wts.numel() < rows * top:
+        raise ValueError("moe_route: buffers shorter than the rows")
+    if experts % groups or not 1 <= keep <= groups or not 1 <= top <= keep * (experts // groups):
+        raise ValueError("moe_route: groups, keep and top do not fit the experts")
+    _check(_fn("bw_moe_route")(logits.data_ptr(), logits.stride(0), rows, experts, top, groups, keep, ids.data_ptr(),
+                               wts.data_ptr(), _stream()), "moe_route")
+
+
+def moe_plan(ids: torch.Tensor, slots: int, experts: int, sorted_slots: torch.Tensor, place: torch.Tensor, tiles: torch.Tensor,
+             meta: torch.Tensor, rank: torch.Tensor) -> None:
+    """The (row, choice) pairs sorted by expert and cut into tiles of one expert each (see moe.hip)."""
+    for t, what in ((ids, "ids"), (sorted_slots, "sorted"), (place, "place"), (tiles, "tiles"), (meta, "meta"), (rank, "rank")):
+        _need(t, torch.int32, what)
+    if min(ids.numel(), sorted_slots.numel(), place.numel(), rank.numel()) < slots or tiles.numel() < 4 * moe_max_tiles(slots, experts) or meta.numel() < 1:
+        raise ValueError("moe_plan: buffers too small")
+    _check(_fn("bw_moe_plan")(ids.data_ptr(), slots, experts, sorted_slots.data_ptr(), place.data_ptr(), tiles.data_ptr(),
+                              meta.data_ptr(), rank.data_ptr(), _stream()), "moe_plan")
+
+
+def moe_experts(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_slots: torch.Tensor, tiles: torch.Tensor,
+                meta: torch.Tensor, slots: int, top: int, gate_up: bool, limit: float = 0.0, alpha: float = 0.0,
+                round_out: bool = False) -> None:
+    """The experts' products over a plan's tiles.  ``gate_up``: x [rows, K] (a slot reads row slot // top), w [experts, 2N, K]
+    (gate rows, then up rows), out [slots, N] = the gated activation by sorted place.  Else: x [slots, K] by sorted place,
+    w [experts, N, K], out [slots, N] float32.  bfloat16 x runs on the matrix cores (bfloat16 weights, K a multiple of 8);
+    float32 x runs 32-bit chains (``round_out``: the activation is rounded to bfloat16 values)."""
+    if w.dim() != 3 or not w.is_cuda or not w.is_contiguous():
+        raise ValueError("moe_experts: weights must be a contiguous [experts, N, K] GPU tensor")
+    experts, N, K = w.shape
+    if gate_up:
+        N //= 2
+    xb, wb = _act_out(x, "x"), _is_bf16(w, "weights")
+    if x.shape[1] != K or out.shape[1] != N or out.shape[0] < slots or (not gate_up and x.shape[0] < slots):
+        raise ValueError("moe_experts: x, w and out do not fit")
+    if xb and (not wb or K % 8):
+        raise ValueError("moe_experts: the matrix-core route takes bfloat16 weights and an inner size that is a multiple of 8")
+    want = torch.bfloat16 if (xb and gate_up) else torch.float32
+    _need(out, want, "out")
+    for t, what in ((sorted_slots, "sorted"), (tiles, "tiles"), (meta, "meta")):
+        _need(t, torch.int32, what)
+    max_tiles = moe_max_tiles(slots, experts)
+    if tiles.numel() < 4 * max_tiles or sorted_slots.numel() < slots:
+        raise ValueError("moe_experts: the plan's tables are too small")
+    _check(_fn("bw_moe_experts")(x.data_ptr(), xb, x.stride(0), w.data_ptr(), wb, out.data_ptr(), out.stride(0), sorted_slots.data_ptr(),
+                                 tiles.data_ptr(), meta.data_ptr(), max_tiles, top, K, N, int(gate_up), float(limit), float(alpha),
+                                 int(round_out), _stream()), "moe_experts")
+
+
+def moe_combine(y: torch.Tensor, place: torch.Tensor, wts: torch.Tensor, top: int, out: torch.Tensor, rows: int,
+                accumulate: bool) -> None:
+    """out[r] (+)= sum_j wts[r, j] * y[place[r*top + j]], j ascending."""
+    _need(y, torch.float32, "y")
+    _need(out, torch.float32, "out")
+    _need(place, torch.int32, "place")
+    _need(wts, torch.float32, "wts")
+    if y.shape[1] != out.shape[1] or out.shape[0] < rows or place.numel() < rows * top or wts.numel() < rows * top:
+        raise ValueError("moe_combine: buffers do not fit")
+    _check(_fn("bw_moe_combine")(y.data_ptr(), y.stride(0), place.data_ptr(), wts.data_ptr(), top, out.data_ptr(), out.stride(0),
+                                 rows, out.shape[1], int(accumulate), _stream()), "moe_combine")
 
 
 # ------------------------------------------------------------------------------ sampling

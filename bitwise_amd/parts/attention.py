@@ -62,6 +62,69 @@ def plan_tiles(ctx, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan
     return ctx.memo(("attention_tiles", tokens_per_tile, group_tiles), make)
 
 
+def _split_scratch(ws, tiles: int, table_width: int, heads: int, kv_heads: int, head_dim: int):
+    """(floats, counters) of the split decode's scratch for this workspace: the worst case over the launches it
+    can see, or (0, 0) if this launch would not split."""
+    if not ops.attention_decode_scratch(tiles, heads, kv_heads, head_dim, table_width, ws.page_size)[0]:
+        return 0, 0
+    width = max(table_width, ws.max_table_width or 0)
+    key = ("attn_split_size", heads, kv_heads, head_dim, width)
+    sizes = ws.notes.get(key)
+    if sizes is None:
+        floats = counters = 0
+        for t in range(1, min(ws.max_rows, 256) + 1):            # (from 256 workgroups on nothing splits)
+            f, c = ops.attention_decode_scratch(t, heads, kv_heads, head_dim, width, ws.page_size)
+            floats, counters = max(floats, f), max(counters, c)
+        sizes = ws.notes[key] = (floats, counters)
+    return sizes
+
+
+def attend_bf16(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, window: int, scale: float, sink=None) -> None:
+    """bfloat16 attention over the call's cache for the step's queries ``q`` [rows, heads*head_dim] into ``out`` (the same
+    shape): prompt portions through the fold kernel, decoded tokens with long contexts through the decode kernel.
+    ``sink`` [heads]: a score per head that joins the denominator and has no value."""
+    ws = ctx.ws
+    table = ctx.block_tables[call.group]
+    tokens_per_tile = 16 // min(heads // kv_heads, 16)
+    plan = plan_tiles(ctx, tokens_per_tile, ops.fold_group_tiles(head_dim))
+    common = (call.k_cache, call.v_cache, out, heads, kv_heads, head_dim, ws.page_size, window, scale)
+    if plan.fold_count:
+        ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common, sink=sink)
+    if plan.decode_count:
+        # few decoded tokens: several workgroups a tile, meeting in device scratch.  One buffer a workspace, sized
+        # for the worst launch it can see (the most tiles that still split, the widest table), whatever this
+        # step's shape: tables grow by a page every few steps, and a buffer per width would pile up.
+        floats, counters = _split_scratch(ws, plan.decode_count, table.stride(0), heads, kv_heads, head_dim)
+        scratch = None
+        if floats:
+            scratch = (ws.buffer("attn_split", floats, torch.float32, rows=1),
+                       ws.buffer("attn_split_count", counters, torch.int32, rows=1))
+        ops.attention_bf16(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, *common, decode=True,
+                           scratch=scratch, sink=sink)
+
+
+def attend_f32(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, window: int, scale: float, sink=None) -> None:
+    """32-bit attention over the call's cache: ``q`` [rows, >= heads*head_dim] with head h at h*head_dim, ``out``
+    [rows, heads*head_dim]."""
+    ws, rows = ctx.ws, ctx.rows
+    table = ctx.block_tables[call.group]
+    # prompt portions: tiles of 32 rows, a wave a tile, both products on the matrix cores; for head sizes
+    # that fill the second product's blocks badly (80 to 112) tiles of 16 rows on the vector units
+    on_matrix_cores = head_dim <= 64 or head_dim == 128
+    plan = plan_tiles(ctx, 32 if on_matrix_cores else 16, 1)
+    common = (call.k_cache, call.v_cache, out, heads, kv_heads, head_dim, ws.page_size, window, scale)
+    if plan.fold_count and head_dim > 128 or (plan.decode_count and plan.decode_tiles is None):
+        # every row by itself (also: a batch of nothing but decoded tokens, row t of request t)
+        ops.attention_f32(q, ctx.positions, ctx.row_seq, table, call.k_cache, call.v_cache, out, rows,
+                          heads, kv_heads, head_dim, ws.page_size, window, scale, sink=sink)
+    else:
+        if plan.fold_count:      # prompt portions: a tile's rows share the keys and values they load
+            ops.attention_f32_tiles(q, ctx.positions, table, plan.fold_tiles, plan.fold_count,
+                                    2 if on_matrix_cores else 1, *common, sink=sink)
+        if plan.decode_count:
+            ops.attention_f32_tiles(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, False, *common, sink=sink)
+
+
 @register_mixer("attention")
 class Attention(Mixer):
     """params: width, heads, kv_heads, head_dim, window (None = all keys), position (PartSpec
@@ -181,60 +244,12 @@ class Attention(Mixer):
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
                              ws.page_size, call.writes_cache)
             out = ws.buffer("attn_out", self.q_dim, torch.float32)
-            # prompt portions: tiles of 32 rows, a wave a tile, both products on the matrix cores; for head sizes
-            # that fill the second product's blocks badly (80 to 112) tiles of 16 rows on the vector units
-            on_matrix_cores = self.head_dim <= 64 or self.head_dim == 128
-            plan = plan_tiles(ctx, 32 if on_matrix_cores else 16, 1)
-            common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, ws.page_size,
-                      window, self.scale)
-            if plan.fold_count and self.head_dim > 128 or (plan.decode_count and plan.decode_tiles is None):
-                # every row by itself (also: a batch of nothing but decoded tokens, row t of request t)
-                ops.attention_f32(qkv, ctx.positions, ctx.row_seq, table, call.k_cache, call.v_cache, out, rows,
-                                  self.heads, self.kv_heads, self.head_dim, ws.page_size, window, self.scale)
-            else:
-                if plan.fold_count:      # prompt portions: a tile's rows share the keys and values they load
-                    ops.attention_f32_tiles(qkv, ctx.positions, table, plan.fold_tiles, plan.fold_count,
-                                            2 if on_matrix_cores else 1, *common)
-                if plan.decode_count:
-                    ops.attention_f32_tiles(qkv, ctx.positions, table, plan.decode_tiles, plan.decode_count, False, *common)
+            attend_f32(ctx, call, qkv, out, self.heads, self.kv_heads, self.head_dim, window, self.scale)
             self.o.add_into(ws, out, residual, rows)
-
-    def _split_scratch(self, ws, tiles: int, table_width: int):
-        """(floats, counters) of the split decode's scratch for this workspace: the worst case over the launches it
-        can see, or (0, 0) if this launch would not split."""
-        if not ops.attention_decode_scratch(tiles, self.heads, self.kv_heads, self.head_dim, table_width, ws.page_size)[0]:
-            return 0, 0
-        width = max(table_width, ws.max_table_width or 0)
-        key = ("attn_split_size", self.heads, self.kv_heads, self.head_dim, width)
-        sizes = ws.notes.get(key)
-        if sizes is None:
-            floats = counters = 0
-            for t in range(1, min(ws.max_rows, 256) + 1):            # (from 256 workgroups on nothing splits)
-                f, c = ops.attention_decode_scratch(t, self.heads, self.kv_heads, self.head_dim, width, ws.page_size)
-                floats, counters = max(floats, f), max(counters, c)
-            sizes = ws.notes[key] = (floats, counters)
-        return sizes
 
     def _attend(self, ctx, call, q, residual) -> None:
         """bfloat16 attention over the cache for rotated queries ``q``, then the output projection."""
-        ws, rows = ctx.ws, ctx.rows
-        table = ctx.block_tables[call.group]
-        window = int(self.window or 0)
+        ws = ctx.ws
         out = ws.buffer("attn_out", self.q_dim, torch.bfloat16)
-        plan = plan_tiles(ctx, self.tokens_per_tile, ops.fold_group_tiles(self.head_dim))
-        common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, ws.page_size,
-                  window, self.scale)
-        if plan.fold_count:
-            ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common)
-        if plan.decode_count:
-            # few decoded tokens: several workgroups a tile, meeting in device scratch.  One buffer a workspace, sized
-            # for the worst launch it can see (the most tiles that still split, the widest table), whatever this
-            # step's shape: tables grow by a page every few steps, and a buffer per width would pile up.
-            floats, counters = self._split_scratch(ws, plan.decode_count, table.stride(0))
-            scratch = None
-            if floats:
-                scratch = (ws.buffer("attn_split", floats, torch.float32, rows=1),
-                           ws.buffer("attn_split_count", counters, torch.int32, rows=1))
-            ops.attention_bf16(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, *common, decode=True,
-                               scratch=scratch)
-        self.o.add_into(ws, out, residual, rows)
+        attend_bf16(ctx, call, q, out, self.heads, self.kv_heads, self.head_dim, int(self.window or 0), self.scale)
+        self.o.add_into(ws, out, residual, ctx.rows)

@@ -22,7 +22,9 @@ class TensorSpec:
 
     kind: "linear" / "embedding" (random init N(0, sigma)), "norm" (1 + N(0, 0.1)),
     "around_zero" (N(0, 0.1): a norm weight stored as its distance from 1), "unit_interval" (a mixing
-    weight in (0, 1)), "bias" (N(0, 1): gate biases, sinks) or "int" (integer table, kept as int32).
+    weight in (0, 1)), "bias" (N(0, 1): gate biases, sinks), "small_bias" (N(0, 0.1)), "conv" (taps of a short convolution,
+    N(0, 0.5)), "router" (N(0, 0.3)), "gate_matrix" (N(0, 1/in): square matrices in front of a sigmoid) or "int" (integer
+    table, kept as int32).
     """
     shape: Tuple[int, ...]
     kind: str = "linear"
@@ -171,6 +173,10 @@ class Norm(Part):
         """x: [rows, width] 32-bit residual stream -> normed rows in the activation dtype."""
         raise NotImplementedError
 
+    def add_normed(self, ctx, y, x) -> None:
+        """x += norm(y), both 32-bit [rows, width]: the norm of a sublayer's output on its way into the residual stream."""
+        raise NotImplementedError
+
 
 class PositionEncoding(Part):
     """Owns its tables; mixers apply it through the kernels they call.
@@ -228,6 +234,14 @@ class Mixer(Part):
         """
         raise NotImplementedError
 
+    def forward_out(self, ctx, call, h, out) -> None:
+        """The mixer's output stored into ``out`` [rows, width] (32-bit) instead of added somewhere: what an
+        arrangement needs that puts something between the mixer and the residual stream (a norm behind the
+        sublayer).  By default the rows are cleared and ``forward`` adds into them; a mixer that can store directly
+        overrides this."""
+        out[:ctx.rows].zero_()
+        self.forward(ctx, call, h, out)
+
     def forward_with_norm(self, ctx, call, x, norm, residual) -> bool:
         """Optional: run ``norm`` and the mixer as fused kernels on the un-normed rows ``x``.
         Return False (and do nothing) if this step cannot be fused; the block then calls the
@@ -243,6 +257,11 @@ class FeedForward(Part):
     def forward(self, ctx, h, residual) -> None:
         """h: normed rows; adds the feed-forward's output into ``residual`` in place."""
         raise NotImplementedError
+
+    def forward_out(self, ctx, h, out) -> None:
+        """As Mixer.forward_out: the output stored into ``out`` instead of added."""
+        out[:ctx.rows].zero_()
+        self.forward(ctx, h, out)
 
 
 class Block(Part):

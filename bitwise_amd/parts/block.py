@@ -2,6 +2,9 @@
 
 from __future__ import annotations
 
+import torch
+
+from ..csrc import ops
 from .base import Block, register_block
 
 
@@ -52,3 +55,35 @@ class ParallelBlock(Block):
                 h2 = self.ffn_norm.forward(ctx, x)
                 self.feed_forward.forward(ctx, h2, x)
         self.mixer.forward(ctx, call, h, x)
+
+
+@register_block("postnorm")
+class PostNormBlock(Block):
+    """x += norm1(mixer(x)); x += norm2(feed_forward(x)): the sublayers read the residual stream itself (in bfloat16
+    mode its rounding, the only rounding between the stream and a sublayer's products), and each sublayer's output is
+    normed on its way back into the stream.  A layer may leave the feed-forward (and its norm) out."""
+
+    roles = {"mixer_norm": "norm", "ffn_norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+    optional_roles = ("ffn_norm", "feed_forward")
+    graph_safe = True
+    launches_through_ops = True
+
+    def __init__(self, parts, runtime):
+        super().__init__(parts, runtime)
+        if (self.feed_forward is None) != (self.ffn_norm is None):
+            raise ValueError("postnorm block: a feed-forward and its norm come together or not at all")
+
+    def _input(self, ctx, x):
+        if not self.rt.bf16:
+            return x
+        h = ctx.ws.buffer("stream_rounded", x.shape[1], torch.bfloat16)
+        ops.convert(x, h, ctx.rows)
+        return h
+
+    def forward(self, ctx, call, x) -> None:
+        y = ctx.ws.buffer("sublayer_out", x.shape[1], torch.float32)
+        self.mixer.forward_out(ctx, call, self._input(ctx, x), y)
+        self.mixer_norm.add_normed(ctx, y, x)
+        if self.feed_forward is not None:
+            self.feed_forward.forward_out(ctx, self._input(ctx, x), y)
+            self.ffn_norm.add_normed(ctx, y, x)

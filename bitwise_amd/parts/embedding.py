@@ -81,3 +81,19 @@ class LMHead(Head):
         normed = norm.forward(ctx, x, out_name="final_normed", rows=count)
         self.linear.store(ws, normed, logits, count)
         return logits
+
+
+@register_head("lm_head_softcap")
+class SoftCappedLMHead(LMHead):
+    """``lm_head`` whose logits are squashed: logits <- cap * tanh(logits / cap), 32-bit, in place.  params as LMHead, plus ``cap``."""
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.cap = float(params["cap"])
+        if not self.cap > 0:
+            raise ValueError("lm_head_softcap: the cap must be positive")
+
+    def forward(self, ctx, x: torch.Tensor, norm, count: int) -> torch.Tensor:
+        logits = super().forward(ctx, x, norm, count)
+        ops.softcap(logits, count, self.cap)
+        return logits

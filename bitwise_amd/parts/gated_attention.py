@@ -1,0 +1,161 @@
+"""Causal grouped-query attention with a short convolution behind its projections, unit-normed rotated queries and
+keys, a sink in the softmax and a gate on its output; a layer may read the keys and values another layer cached.
+
+    q, k, v = conv(W_q h), conv(W_k h), conv(W_v h)       a causal convolution over `taps` tokens per channel
+    q, k    = unit(rot(q)), unit(rot(k))                   pairs (2i, 2i+1) of the first rot elements turned by the
+                                                           position's angles, then x / sqrt(mean(x^2) + eps) per head
+    p_j     = exp(s_j) / (exp(sink) + sum_i exp(s_i))      s_j = scale * q . k_j over the keys j <= the query's position
+    out     = W_o ((sum_j p_j v_j) * sigmoid(W_g h))
+
+Every step is switched by a parameter, so that another design can take what it needs: ``conv`` (taps; 0 or 1 with no
+convolution tensor: none), ``qk_norm``, ``sink`` (None, or a number that every head uses), ``gate``, ``shared_kv``
+(no key and value tensors: the call reads the cache of the layer the schedule names), query/key size ``dim`` and value
+size ``vdim`` (the cache's head size is the larger of the two, rounded up to what the attention kernels take; the
+padding is zeros).  The last taps - 1 projected rows of a request are its state.  Convolution, rotation, norms, scores
+and softmax are 32-bit in both modes; the cache, the queries and the gated output have the mode's activation dtype.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..csrc import ops
+from .attention import attend_bf16, attend_f32
+from .base import CacheSpec, Mixer, StateSpec, TensorSpec, lookup, register_mixer, POSITION_ENCODINGS
+from .linear import Linear
+
+
+def max_seq_rows(ctx) -> int:
+    """The most rows one request brings in this step."""
+    if getattr(ctx, "one_row_per_request", False):
+        return 1
+    return ctx.memo(("max_seq_rows",), lambda: max(len(s.tokens) for s in ctx.segments))
+
+
+@register_mixer("gated_attention")
+class GatedAttention(Mixer):
+    """params: width, heads, kv_heads, dim, vdim, scale, eps, conv (taps), qk_norm, sink, gate, shared_kv, window,
+    position (PartSpec of a position encoding with the layout "pairs").
+    tensors: q, k, v [heads*dim | kv_heads*dim | kv_heads*vdim, width]; q.conv, k.conv, v.conv [channels, taps];
+    g [heads*vdim, width]; o [width, heads*vdim]."""
+
+    graph_safe = True
+    launches_through_ops = True
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        p = params
+        self.width, self.heads, self.kv_heads = int(p["width"]), int(p["heads"]), int(p["kv_heads"])
+        self.dim, self.vdim = int(p["dim"]), int(p["vdim"])
+        self.scale, self.eps = float(p["scale"]), float(p.get("eps", 0.0))
+        self.taps = int(p.get("conv") or 0)
+        self.qk_norm, self.gate, self.shared_kv = bool(p.get("qk_norm", False)), bool(p.get("gate", False)), bool(p.get("shared_kv", False))
+        self.sink_value: Optional[float] = None if p.get("sink") is None else float(p["sink"])
+        self.window: Optional[int] = p.get("window")
+        if self.heads % self.kv_heads:
+            raise ValueError(f"gated_attention: {self.heads} heads are no multiple of {self.kv_heads} kv heads")
+        if not self.scale > 0:
+            raise ValueError("gated_attention: the score scale must be positive")
+        if self.taps > ops.CONV_MAX_TAPS:
+            raise ValueError(f"gated_attention: a convolution over {self.taps} tokens; the kernel takes up to {ops.CONV_MAX_TAPS}")
+        need = max(self.dim, self.vdim)
+        fits = [d for d in ops.HEAD_DIMS if d >= need]
+        if not fits:
+            raise ValueError(f"gated_attention: heads of {need} elements; the attention kernels take up to {ops.HEAD_DIMS[-1]}")
+        self.head_size = fits[0]                       # the cache's head size
+        pos = p["position"]
+        self.position = lookup(POSITION_ENCODINGS, "position encoding", pos.kind).shared(pos.params, runtime)
+        if getattr(self.position, "layout", None) != "pairs":
+            raise ValueError(f"gated_attention rotates neighbouring pairs; position encoding '{pos.kind}' is laid out otherwise")
+        self.rot = int(self.position.rotary_dim)
+        if self.rot > self.dim:
+            raise ValueError(f"gated_attention: {self.rot} rotated elements in heads of {self.dim}")
+        self.q_ch = self.heads * self.dim
+        self.kv_ch = 0 if self.shared_kv else self.kv_heads * (self.dim + self.vdim)
+        self.conv_ch = self.q_ch + self.kv_ch
+        self.g_ch = self.heads * self.vdim if self.gate else 0
+        self.proj: Optional[Linear] = None
+        self.o: Optional[Linear] = None
+        self.conv_w = self.sink = self.cos = self.sin = None
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        out = {"q": TensorSpec((self.q_ch, self.width))}
+        if not self.shared_kv:
+            out["k"] = TensorSpec((self.kv_heads * self.dim, self.width))
+            out["v"] = TensorSpec((self.kv_heads * self.vdim, self.width))
+        if self.taps >= 1:
+            out["q.conv"] = TensorSpec((self.q_ch, self.taps), "conv")
+            if not self.shared_kv:
+                out["k.conv"] = TensorSpec((self.kv_heads * self.dim, self.taps), "conv")
+                out["v.conv"] = TensorSpec((self.kv_heads * self.vdim, self.taps), "conv")
+        if self.gate:
+            out["g"] = TensorSpec((self.g_ch, self.width))
+        out["o"] = TensorSpec((self.width, self.heads * self.vdim))
+        return out
+
+    def bind(self, tensors) -> None:
+        self.cos, self.sin = self.position.tables()
+        names = ["q"] + ([] if self.shared_kv else ["k", "v"]) + (["g"] if self.gate else [])
+        stack = [tensors[n] for n in names]
+        if len({t.dtype for t in stack}) != 1:
+            raise ValueError("the projections of one mixer must be stored in one dtype to be stacked")
+        self.proj = Linear(torch.cat(stack, dim=0), self.rt)
+        self.o = Linear(tensors["o"], self.rt)
+        dev = self.rt.device
+        if self.taps >= 1:
+            cn = ["q.conv"] + ([] if self.shared_kv else ["k.conv", "v.conv"])
+            self.conv_w = torch.cat([tensors[n].to(dev).float() for n in cn], dim=0).contiguous()      # (widening is exact)
+        if self.sink_value is not None:
+            self.sink = torch.full((self.heads,), self.sink_value, dtype=torch.float32, device=dev)
+
+    def weight_bytes(self) -> int:
+        return self.proj.nbytes() + self.o.nbytes() + (0 if self.conv_w is None else self.conv_w.numel() * 4)
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(self.kv_heads, self.head_size, self.window)
+
+    def page_sizes(self):
+        return ops.PAGE_SIZES
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return StateSpec(((self.taps - 1) * self.conv_ch,), "float32") if self.taps > 1 else None
+
+    def _run(self, ctx, call, h, target, add: bool) -> None:
+        rt, ws, rows = self.rt, ctx.ws, ctx.rows
+        if self.shared_kv == bool(call.writes_cache):
+            raise ValueError("gated_attention: a layer with keys and values of its own writes its cache, one without reads another's")
+        proj = ws.buffer("gattn_proj", self.proj.out_features, torch.float32)
+        self.proj.store(ws, h, proj, rows)
+        src = proj
+        if self.taps >= 1:
+            src = ws.buffer("gattn_conv", self.conv_ch, torch.float32)
+            ops.causal_conv(proj, self.conv_w, None, call.state, ctx.seq_rows, ctx.slots, ctx.positions, ctx.nseq,
+                            max_seq_rows(ctx), src)
+        hs = self.head_size
+        q = ws.buffer("gattn_q", self.heads * hs, rt.act_dtype)
+        ops.pair_rope_unit(src, ctx.positions, ctx.row_seq, ctx.block_tables[call.group], self.cos, self.sin, q, call.k_cache,
+                           call.v_cache, rows, self.heads, self.kv_heads, self.dim, self.vdim, hs, self.rot, ws.page_size,
+                           self.qk_norm, self.eps, not self.shared_kv, call.writes_cache)
+        av = ws.buffer("gattn_av", self.heads * hs, rt.act_dtype)
+        attend = attend_bf16 if rt.bf16 else attend_f32
+        attend(ctx, call, q, av, self.heads, self.kv_heads, hs, int(self.window or 0), self.scale, sink=self.sink)
+        if self.gate or hs != self.vdim:
+            act = ws.buffer("gattn_gated", self.heads * self.vdim, rt.act_dtype)
+            if self.gate:
+                ops.gate_mul(av, hs, proj[:, self.conv_ch:], act, rows, self.heads, self.vdim)
+            else:
+                act.view(-1, self.heads, self.vdim)[:rows].copy_(av.view(-1, self.heads, hs)[:rows, :, :self.vdim])
+        else:
+            act = av
+        if add:
+            self.o.add_into(ws, act, target, rows)
+        else:
+            self.o.store(ws, act, target, rows)
+
+    def forward(self, ctx, call, h, residual) -> None:
+        self._run(ctx, call, h, residual, True)
+
+    def forward_out(self, ctx, call, h, out) -> None:
+        self._run(ctx, call, h, out, False)

@@ -1,0 +1,105 @@
+"""A feed-forward of routed experts: every row goes through the ``top`` experts its router scores pick, and their
+outputs are added with the scores as weights.
+
+    s       = softmax(W_router h)                              over all experts, 32-bit
+    allowed = the experts of the `keep` best of `groups` equal groups of neighbours (a group's score: its best expert's)
+    chosen  = the `top` allowed experts with the largest s; weights = their s, as they are
+    expert  : g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), W_down (g sigmoid(alpha g) (u + 1))
+
+Routing happens on the device and the experts' products run over a plan built there, so a step never waits for the
+host and a captured decode step stays valid.  What a row gets from an expert depends on the row and the expert
+alone, whatever else is in the batch.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..csrc import ops
+from .base import FeedForward, TensorSpec, register_feed_forward
+from .linear import Linear
+
+
+@register_feed_forward("moe")
+class RoutedExperts(FeedForward):
+    """params: width, experts, top, groups (1), keep (groups), ff, limit, alpha (1.702).
+    tensors: router [experts, width]; e<j>.gate, e<j>.up [ff, width]; e<j>.down [width, ff]."""
+
+    graph_safe = True
+    launches_through_ops = True
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        p = params
+        self.width, self.experts, self.top, self.ff = int(p["width"]), int(p["experts"]), int(p["top"]), int(p["ff"])
+        self.groups = int(p.get("groups", 1))
+        self.keep = int(p.get("keep", self.groups))
+        self.limit, self.alpha = float(p["limit"]), float(p.get("alpha", 1.702))
+        if self.experts % self.groups or not 1 <= self.keep <= self.groups:
+            raise ValueError(f"moe: {self.experts} experts in {self.groups} groups of which {self.keep} are kept")
+        if not 1 <= self.top <= self.keep * (self.experts // self.groups):
+            raise ValueError(f"moe: {self.top} experts a row out of {self.keep} groups of {self.experts // self.groups}")
+        self.router: Optional[Linear] = None
+        self.gate_up = self.down = None
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        out = {}
+        for j in range(self.experts):
+            out[f"e{j}.gate"] = TensorSpec((self.ff, self.width))
+            out[f"e{j}.up"] = TensorSpec((self.ff, self.width))
+            out[f"e{j}.down"] = TensorSpec((self.width, self.ff))
+        out["router"] = TensorSpec((self.experts, self.width), "router")
+        return out
+
+    def bind(self, tensors) -> None:
+        dev = self.rt.device
+        # the router's product stays 32-bit in either mode
+        self.router = Linear(tensors["router"], self.rt, matrix_cores=False)
+        kinds = {tensors[f"e{j}.{n}"].dtype for j in range(self.experts) for n in ("gate", "up", "down")}
+        if len(kinds) != 1:
+            raise ValueError("the experts of one feed-forward must be stored in one dtype to be stacked")
+        self.gate_up = torch.stack([torch.cat([tensors[f"e{j}.gate"], tensors[f"e{j}.up"]], dim=0) for j in range(self.experts)]).to(dev).contiguous()
+        self.down = torch.stack([tensors[f"e{j}.down"] for j in range(self.experts)]).to(dev).contiguous()
+        self.mfma = bool(self.rt.bf16 and self.gate_up.dtype == torch.bfloat16 and self.width % 8 == 0 and self.ff % 8 == 0)
+
+    def weight_bytes(self) -> int:
+        """Bytes a decode step of one row reads: the router and the chosen experts."""
+        per = (self.gate_up.numel() + self.down.numel()) // self.experts * self.gate_up.element_size()
+        return self.router.nbytes() + self.top * per
+
+    def _run(self, ctx, h, target, add: bool) -> None:
+        rt, ws, rows = self.rt, ctx.ws, ctx.rows
+        slots = rows * self.top
+        most = ws.max_rows * self.top
+        logits = ws.buffer("moe_logits", self.experts, torch.float32)
+        self.router.store(ws, h, logits, rows)
+        ids = ws.buffer("moe_ids", self.top, torch.int32)
+        wts = ws.buffer("moe_wts", self.top, torch.float32)
+        ops.moe_route(logits, rows, self.top, self.groups, self.keep, ids, wts)
+        sorted_slots = ws.buffer("moe_sorted", most, torch.int32, rows=1)
+        place = ws.buffer("moe_place", most, torch.int32, rows=1)
+        rank = ws.buffer("moe_rank", most, torch.int32, rows=1)
+        tiles = ws.buffer("moe_tiles", 4 * ops.moe_max_tiles(most, self.experts), torch.int32, rows=1)
+        meta = ws.buffer("moe_meta", 4, torch.int32, rows=1)
+        ops.moe_plan(ids, slots, self.experts, sorted_slots, place, tiles, meta, rank)
+        if self.mfma:
+            x, act_dtype = h, torch.bfloat16
+        else:
+            x, act_dtype = h, torch.float32
+            if h.dtype != torch.float32:
+                x = ws.buffer("moe_x32", self.width, torch.float32)
+                ops.convert(h, x, rows)
+        act = ws.buffer("moe_act", self.ff, act_dtype, rows=most)
+        ops.moe_experts(x, self.gate_up, act, sorted_slots, tiles, meta, slots, self.top, True, self.limit, self.alpha,
+                        round_out=rt.bf16 and not self.mfma)
+        y = ws.buffer("moe_y", self.width, torch.float32, rows=most)
+        ops.moe_experts(act, self.down, y, sorted_slots, tiles, meta, slots, self.top, False)
+        ops.moe_combine(y, place, wts, self.top, target, rows, add)
+
+    def forward(self, ctx, h, residual) -> None:
+        self._run(ctx, h, residual, True)
+
+    def forward_out(self, ctx, h, out) -> None:
+        self._run(ctx, h, out, False)

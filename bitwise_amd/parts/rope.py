@@ -51,3 +51,65 @@ class RotaryTable(PositionEncoding):
     def shared(cls, params, runtime) -> "RotaryTable":
         key = ("rope", float(params["theta"]), int(params["head_dim"]), int(params["max_positions"]))
         return runtime.shared(key, lambda: cls(params, runtime))
+
+
+@register_position_encoding("rope_pairs")
+class PairRotaryTable(PositionEncoding):
+    """Rotary angles for mixers that rotate neighbouring pairs (2i, 2i+1) of a head's first ``dims`` elements:
+    angle = position * f_i, f_i = base^(-2i/dims), optionally stretched band by band.
+
+    params: base, dims, max_positions; optional ``scaling`` = {factor, low, high, original}: with the wavelength
+    l = 2 pi / f, a frequency stays where l < original / high, becomes f / factor where l > original / low, and in
+    between is (1 - s) f / factor + s f with s = (original / l - low) / (high - low).
+    Frequencies and angles are computed in double precision on the host and the cosines and sines rounded once to
+    32-bit.  No checkpoint tensors.  The tables are those of the base contract, [positions, dims / 2]; which
+    elements a column pairs is the mixer's business (``layout``)."""
+
+    graph_safe = True
+    launches_through_ops = True
+    layout = "pairs"
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.base = float(params["base"])
+        self.rotary_dim = int(params["dims"])
+        self.max_positions = int(params["max_positions"])
+        self.scaling = dict(params["scaling"]) if params.get("scaling") else None
+        if self.rotary_dim % 2 or self.rotary_dim < 0:
+            raise ValueError("rotary encoding needs an even number of rotated elements")
+        if self.scaling is not None:
+            missing = [k for k in ("factor", "low", "high", "original") if k not in self.scaling]
+            if missing:
+                raise ValueError(f"rope_pairs: scaling lacks {missing}")
+            if float(self.scaling["high"]) == float(self.scaling["low"]):
+                raise ValueError("rope_pairs: scaling needs high != low")
+        self._cos = self._sin = None
+
+    def frequencies(self) -> np.ndarray:
+        half = self.rotary_dim // 2
+        f = np.power(np.float64(self.base), -2.0 * np.arange(half, dtype=np.float64) / max(self.rotary_dim, 1))
+        sc = self.scaling
+        if sc is None:
+            return f
+        factor, low, high, orig = (float(sc[k]) for k in ("factor", "low", "high", "original"))
+        wavelength = 2.0 * np.pi / f
+        blend = (orig / wavelength - low) / (high - low)
+        mixed = (1.0 - blend) * f / factor + blend * f
+        return np.where(wavelength < orig / high, f, np.where(wavelength > orig / low, f / factor, mixed))
+
+    def _build(self) -> None:
+        angle = np.arange(self.max_positions, dtype=np.float64)[:, None] * self.frequencies()[None, :]
+        self._cos = torch.from_numpy(np.cos(angle).astype(np.float32)).to(self.rt.device).contiguous()
+        self._sin = torch.from_numpy(np.sin(angle).astype(np.float32)).to(self.rt.device).contiguous()
+
+    def tables(self):
+        if self._cos is None:
+            self._build()
+        return self._cos, self._sin
+
+    @classmethod
+    def shared(cls, params, runtime) -> "PairRotaryTable":
+        sc = params.get("scaling")
+        key = ("rope_pairs", float(params["base"]), int(params["dims"]), int(params["max_positions"]),
+               None if not sc else tuple(sorted((k, float(v)) for k, v in sc.items())))
+        return runtime.shared(key, lambda: cls(params, runtime))

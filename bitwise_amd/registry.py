@@ -10,9 +10,11 @@ from pathlib import Path
 from typing import Any, Callable, Dict, Mapping, Optional
 
 from .config import kuponex as kuponex_config
+from .config import sepedra as sepedra_config
 from .config.llama import ConfigError, LlamaConfig
 from .models.kuponex import TINY_KUPONEX, kuponex_spec
 from .models.llama import TINY_LLAMA, llama_spec
+from .models.sepedra import TINY_SEPEDRA, sepedra_spec
 from .parts.base import ModelSpec
 
 
@@ -75,3 +77,4 @@ def read_config(folder: str | Path) -> Dict[str, Any]:
 register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec, TINY_LLAMA)
 register_architecture(kuponex_config.ARCHITECTURE, kuponex_config.KuponexConfig.from_dict, kuponex_spec, TINY_KUPONEX,
                       kuponex_config.sizes_from_tensors)
+register_architecture(sepedra_config.ARCHITECTURE, sepedra_config.SepedraConfig.from_dict, sepedra_spec, TINY_SEPEDRA)

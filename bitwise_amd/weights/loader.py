@@ -93,6 +93,14 @@ def shape_values(kind: str, z: torch.Tensor, sigma: float) -> torch.Tensor:
         return torch.sigmoid(z)
     if kind == "bias":
         return z
+    if kind == "small_bias":
+        return 0.1 * z
+    if kind == "conv":                         # taps of a short convolution: of the order of 1 / taps
+        return 0.5 * z
+    if kind == "router":                       # logits that spread over a few units
+        return 0.3 * z
+    if kind == "gate_matrix":                  # square matrices in front of a sigmoid: rows of norm about 1 for inputs of norm 1
+        return z / (z.shape[-1] ** 0.5)
     return sigma * z
 
 
