@@ -85,11 +85,12 @@ def attend_bf16(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, win
     ``sink`` [heads]: a score per head that joins the denominator and has no value."""
     ws = ctx.ws
     table = ctx.block_tables[call.group]
+    extra = {} if sink is None else {"sink": sink}
     tokens_per_tile = 16 // min(heads // kv_heads, 16)
     plan = plan_tiles(ctx, tokens_per_tile, ops.fold_group_tiles(head_dim))
     common = (call.k_cache, call.v_cache, out, heads, kv_heads, head_dim, ws.page_size, window, scale)
     if plan.fold_count:
-        ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common, sink=sink)
+        ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common, **extra)
     if plan.decode_count:
         # few decoded tokens: several workgroups a tile, meeting in device scratch.  One buffer a workspace, sized
         # for the worst launch it can see (the most tiles that still split, the widest table), whatever this
@@ -100,7 +101,7 @@ def attend_bf16(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, win
             scratch = (ws.buffer("attn_split", floats, torch.float32, rows=1),
                        ws.buffer("attn_split_count", counters, torch.int32, rows=1))
         ops.attention_bf16(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, *common, decode=True,
-                           scratch=scratch, sink=sink)
+                           scratch=scratch, **extra)
 
 
 def attend_f32(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, window: int, scale: float, sink=None) -> None:
@@ -108,6 +109,7 @@ def attend_f32(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, wind
     [rows, heads*head_dim]."""
     ws, rows = ctx.ws, ctx.rows
     table = ctx.block_tables[call.group]
+    extra = {} if sink is None else {"sink": sink}
     # prompt portions: tiles of 32 rows, a wave a tile, both products on the matrix cores; for head sizes
     # that fill the second product's blocks badly (80 to 112) tiles of 16 rows on the vector units
     on_matrix_cores = head_dim <= 64 or head_dim == 128
@@ -116,13 +118,13 @@ def attend_f32(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, wind
     if plan.fold_count and head_dim > 128 or (plan.decode_count and plan.decode_tiles is None):
         # every row by itself (also: a batch of nothing but decoded tokens, row t of request t)
         ops.attention_f32(q, ctx.positions, ctx.row_seq, table, call.k_cache, call.v_cache, out, rows,
-                          heads, kv_heads, head_dim, ws.page_size, window, scale, sink=sink)
+                          heads, kv_heads, head_dim, ws.page_size, window, scale, **extra)
     else:
         if plan.fold_count:      # prompt portions: a tile's rows share the keys and values they load
             ops.attention_f32_tiles(q, ctx.positions, table, plan.fold_tiles, plan.fold_count,
-                                    2 if on_matrix_cores else 1, *common, sink=sink)
+                                    2 if on_matrix_cores else 1, *common, **extra)
         if plan.decode_count:
-            ops.attention_f32_tiles(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, False, *common, sink=sink)
+            ops.attention_f32_tiles(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, False, *common, **extra)
 
 
 @register_mixer("attention")

@@ -204,3 +204,25 @@ def forward(cfg: Mapping, w: Mapping[str, torch.Tensor], tokens, rnd=identity, l
     cap = float(cfg["logit_softcap"])
     logits = rnd(rms_norm(x, w["final.norm"], eps)) @ w["head"].T
     return cap * torch.tanh(logits / cap)
+
+
+def generate_greedy(cfg: Mapping, w: Mapping[str, torch.Tensor], prompt, n: int) -> List[int]:
+    """n tokens by the first maximum of the last position's logits, the whole sequence recomputed for every token."""
+    toks = list(prompt)
+    out: List[int] = []
+    for _ in range(n):
+        nxt = int(torch.argmax(forward(cfg, w, toks)[-1]))
+        out.append(nxt)
+        toks.append(nxt)
+    return out
+
+
+def logits_error(got, want, quantile: float = 1.0) -> float:
+    """A row's error: the root mean square of the difference (its mean taken off) over that of the wanted row; the
+    largest over the rows, or the given quantile of them."""
+    import numpy as np
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    ref = want - want.mean(-1, keepdims=True)
+    return float(np.quantile(np.sqrt((d * d).mean(-1)) / np.sqrt((ref * ref).mean(-1)), quantile))
