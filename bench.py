@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep] [--kuponex]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep] [--kuponex] [--sepedra]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -99,6 +99,48 @@ def kuponex_comparison(bw, torch, steps: int, dtype: str, only: str = "") -> int
     return 0
 
 
+def sepedra_shape(width: int, expert_ff: int, groups: int, experts: int = 32, top: int = 4, vocab: int = 32000) -> dict:
+    """A Sepedra of ``groups`` x (two recurrent layers, an attention layer, an attention layer that reads the first one's
+    cache), heads of 128 with a quarter as many key heads, recurrent branches as wide as the model in blocks of 128,
+    feed-forwards of ``experts`` experts of which a token uses ``top``."""
+    heads = width // 128
+    rot = {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    mlp = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0},
+           "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}
+    layers = []
+    for g in range(groups):
+        for _ in range(2):
+            layers.append({"type": "rglru", "mixer": {"width": width, "blocks": heads, "conv": 4}, "mlp": mlp})
+        att = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5, "rot": rot}
+        layers.append({"type": "attention", "mixer": dict(att), "mlp": mlp})
+        layers.append({"type": "attention", "mixer": dict(att, kv_from=4 * g + 2), "mlp": mlp})
+    return {"architecture": "Sepedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "layers": layers, "max_positions": 16384, "eos_token_id": 2}
+
+
+def sepedra_comparison(bw, torch, steps: int, dtype: str, only: str = "") -> int:
+    """Prefill and decode of Sepedra at two layer sizes beside the Llama decoder of equal width and depth whose
+    feed-forward is as wide as the experts a token uses together: one JSON object a line."""
+    from bitwise_amd.measure import PEAK_FLOPS, measure_decode, measure_prefill
+    for name, width, expert_ff, groups in (("2048x(4x2048 of 32)", 2048, 2048, 2), ("4096x(4x3584 of 32)", 4096, 3584, 2)):
+        for arch, cfg in (("Sepedra", sepedra_shape(width, expert_ff, groups)), ("Llama", llama_shape(width, 4 * expert_ff, 4 * groups))):
+            if only and only.lower() != arch.lower():
+                continue
+            model = bw.Model.random(cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
+            for tokens in (512, 2048):
+                m = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[dtype], tokens)
+                print(json.dumps({"shape": name, "model": arch, "dtype": dtype, "prefill_tokens": tokens,
+                                  "ms": m["ms"], "tok_s": m["value"], "frac_of_matrix_peak": m["frac"]}), flush=True)
+            for batch in (1, 8, 64):
+                m = measure_decode(bw, torch, model, cfg, dtype, batch, steps, 4, context=2048)
+                print(json.dumps({"shape": name, "model": arch, "dtype": dtype, "decode_batch": batch, "context": 2048,
+                                  "ms_per_step": m["ms_per_step"], "tok_s": m["tok_s"], "frac_of_8_TBs": m["roofline"]["frac"]}),
+                      flush=True)
+            del model
+            torch.cuda.empty_cache()
+    return 0
+
+
 def sweep(bw, torch, steps: int, dtype: str) -> int:
     """Decode steps over batch and context, prefills over length: in bfloat16 at both shapes, in the 32-bit mode a
     coarser grid at the small one.  One JSON object a line."""
@@ -148,6 +190,9 @@ def main() -> int:
     ap.add_argument("--sweep", action="store_true",
                     help="print a table instead of the line: decode at batches 1 to 128 and contexts of 512 to 8,192 tokens, prefills "
                          "of 128 to 2,048 tokens, at both shapes (with --dtype fp32: a coarser grid at the small shape)")
+    ap.add_argument("--sepedra", nargs="?", const="both", default="", choices=["both", "sepedra", "llama"],
+                    help="print a table instead of the line: prefill and decode of the Sepedra design at two layer sizes beside "
+                         "the Llama decoder of equal width and depth with a feed-forward as wide as a token's experts together")
     ap.add_argument("--kuponex", nargs="?", const="both", default="", choices=["both", "kuponex", "llama"],
                     help="print a table instead of the line: prefill and decode of the Kuponex design at two layer sizes beside "
                          "the Llama decoder of equal width, depth and feed-forward (or only one of the two)")
@@ -166,6 +211,8 @@ def main() -> int:
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     if args.sweep:
         return sweep(bw, torch, args.steps, dtype)
+    if args.sepedra:
+        return sepedra_comparison(bw, torch, min(args.steps, 32), dtype, "" if args.sepedra == "both" else args.sepedra)
     if args.kuponex:
         return kuponex_comparison(bw, torch, min(args.steps, 32), dtype, "" if args.kuponex == "both" else args.kuponex)
     if args.mixed:

@@ -40,9 +40,33 @@ def kuponex_prefill_flops(cfg: dict, tokens: int) -> float:
     return total + 2 * w * cfg["vocab"]
 
 
+def sepedra_prefill_flops(cfg: dict, tokens: int) -> float:
+    """Multiply-adds times two of one prompt: every projection, the gates' block-diagonal products, the router and the
+    chosen experts, and the attention's scores and weighted sums (the convolutions and the recurrence itself are a few
+    operations a channel and are left out)."""
+    w, total = cfg["width"], 0.0
+    for layer in cfg["layers"]:
+        m, per_token, quadratic = layer["mixer"], 0.0, 0.0
+        if layer["type"] == "attention":
+            H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            own = 0 if m.get("kv_from") is not None else G * (D + V)
+            per_token = w * (H * D + own + H * V) + H * V * w
+            quadratic = H * (D + V) * tokens * (tokens + 1) / 2
+        else:
+            R = m["width"]
+            per_token = w * 2 * R + 2 * R * (R // m["blocks"]) + R * w
+        if layer.get("mlp"):
+            ro, ex = layer["mlp"]["router"], layer["mlp"]["expert"]
+            per_token += w * ro["experts"] + ro["top"] * 3 * w * ex["ff"]
+        total += 2 * (per_token * tokens + quadratic)
+    return total + 2 * w * cfg["vocab"]
+
+
 def prefill_flops(cfg: dict, tokens: int) -> float:
     if cfg.get("architecture") == "Kuponex":
         return kuponex_prefill_flops(cfg, tokens)
+    if cfg.get("architecture") == "Sepedra":
+        return sepedra_prefill_flops(cfg, tokens)
     h, inter, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     qd = cfg["num_attention_heads"] * cfg["head_dim"]
     kvd = cfg["num_key_value_heads"] * cfg["head_dim"]
@@ -246,7 +270,8 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
     # keys a decoded token reads, on average: the prompt, what the request decoded while later
     # prompts were prefilled, the warm-up, and half the timed steps
     avg_ctx = context + batch * context / 2048 * (batch - 1) / (2 * batch) + warmup + (steps + 1) / 2
-    step_bytes = model.weight_bytes + batch * avg_ctx * kv_token + 2 * batch * slot_bytes
+    # (a model of routed experts reads the experts its rows choose: what a step of ``batch`` rows reads on average)
+    step_bytes = model.weight_bytes_for(batch) + batch * avg_ctx * kv_token + 2 * batch * slot_bytes
     achieved = step_bytes / (ms * 1e-3) / 1e9
     return {"tok_s": round(batch * steps / secs, 1), "ms_per_step": round(ms, 4),
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

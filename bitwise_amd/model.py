@@ -102,6 +102,10 @@ class Model:
     def weight_bytes(self) -> int:
         return self.assembled.weight_bytes()
 
+    def weight_bytes_for(self, rows: int) -> int:
+        """Bytes of weights a decode step of ``rows`` rows reads (parts that read only what their rows choose say how much)."""
+        return self.assembled.weight_bytes(rows)
+
     # ------------------------------------------------------------------ numerics entry
     def logits(self, tokens: Sequence[int], chunk: Optional[int] = None, block_size: int = 16) -> np.ndarray:
         """Logits [n, vocab] at every position of one sequence, run as a prompt through a

@@ -142,12 +142,15 @@ class AssembledModel:
             else:
                 part.bind(mine)
 
-    def weight_bytes(self) -> int:
-        """Bytes of weights one decode step reads: every layer call's weights once, the final
-        norm and the head (a tied head is the embedding table, read whole as the head)."""
+    def weight_bytes(self, rows: int = 1) -> int:
+        """Bytes of weights one decode step of ``rows`` rows reads: every layer call's weights once, the final
+        norm and the head (a tied head is the embedding table, read whole as the head).  A part that reads only what
+        its rows choose (routed experts) says how much that is for so many rows (``weight_bytes_rows``)."""
         total = self.final_norm.weight_bytes() + self.lm_head.weight_bytes()
         for call in self.calls:
-            total += sum(p.weight_bytes() for p in self.layers[call.layer].parts.values())
+            for p in self.layers[call.layer].parts.values():
+                by_rows = getattr(p, "weight_bytes_rows", None)
+                total += p.weight_bytes() if by_rows is None else by_rows(rows)
         return total
 
     # ------------------------------------------------------------------ forward

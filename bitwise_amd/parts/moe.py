@@ -69,6 +69,13 @@ class RoutedExperts(FeedForward):
         per = (self.gate_up.numel() + self.down.numel()) // self.experts * self.gate_up.element_size()
         return self.router.nbytes() + self.top * per
 
+    def weight_bytes_rows(self, rows: int) -> int:
+        """Bytes a decode step of ``rows`` rows reads: the router and the experts the rows touch, on average, if every
+        expert is as likely as any other: experts * (1 - (1 - top/experts)^rows)."""
+        per = (self.gate_up.numel() + self.down.numel()) // self.experts * self.gate_up.element_size()
+        touched = self.experts * (1.0 - (1.0 - self.top / self.experts) ** max(int(rows), 1))
+        return self.router.nbytes() + int(touched * per)
+
     def _run(self, ctx, h, target, add: bool) -> None:
         rt, ws, rows = self.rt, ctx.ws, ctx.rows
         slots = rows * self.top
