@@ -137,19 +137,20 @@ int bw_pair_rope_unit(const float* src, int lds, const int32_t* positions, const
                       int write_cache, void* stream);
 int bw_gate_mul(const void* av, int a_is_bf16, int lda, int hd, const float* g, int ldg, void* out, int out_is_bf16,
                 int ldo, int rows, int heads, int vdim, void* stream);
-int bw_rglru_scan(const float* y, int ldy, const float* u, int ldu, const float* gates, int ldg, const float* ra_bias,
+// (y and gates are overwritten: y by its activation, the gates' logits by the recurrence's factor and addend)
+int bw_rglru_scan(float* y, int ldy, const float* u, int ldu, float* gates, int ldg, const float* ra_bias,
                   const float* ri_bias, const float* decay, float* state, long long state_ld, void* out,
                   int out_is_bf16, int ldo, const int32_t* seq_rows, const int32_t* slots, const int32_t* positions,
-                  int nseq, int channels, int bs, void* stream);
-int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, int rows, int dim, float eps,
-                void* stream);
+                  int nseq, int rows, int channels, int bs, void* stream);
+int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, void* rounded, int ldr,
+                int rows, int dim, float eps, void* stream);
 int bw_softcap(float* x, int ld, int rows, int cols, float cap, void* stream);
 // A feed-forward of routed experts (moe.hip).
 int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
                  float* wts, void* stream);
 int bw_moe_max_tiles(int slots, int experts);
 int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* sorted, int32_t* place, int32_t* tiles,
-                int32_t* meta, int32_t* rank, void* stream);
+                int32_t* meta, void* stream);
 int bw_moe_experts(const void* x, int x_is_bf16, int ldx, const void* w, int w_is_bf16, void* out, int ldo,
                    const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int max_tiles, int top, int K,
                    int N, int gate_up, float limit, float alpha, int round_out, void* stream);

@@ -9,7 +9,7 @@
 //   gate_mul:      out = a * sigmoid(g), heads compacted from the attention's head size to the value size
 //   rglru_scan:    S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t with a_t = exp(c r_t), r and i sigmoids of block-diagonal
 //                  projections of u; out = S_t * gelu_tanh(y_t)
-//   norm_add:      x += y / sqrt(mean(y^2) + eps) * w
+//   norm_add:      x += y / sqrt(mean(y^2) + eps) * w (and, if asked, the new x once more rounded to bfloat16)
 //   softcap:       x = cap * tanh(x / cap)
 //
 // All arithmetic is 32-bit; only stores into a bfloat16 buffer round.  A request without rows, with a negative slot or
@@ -282,55 +282,65 @@ __device__ __forceinline__ void rglru_terms(float zr, float zi, float u, float b
   b = sqrtf(-expm1f(2.0f * log_a)) * (i * u);      // sqrt(1 - a^2) without the cancellation near a = 1
 }
 
+// Pass 1, a thread an element (row, channel): the factor a, the addend b and the gate branch's activation, each a
+// function of the row alone, over the gates' logits, u and y in place (gates[.., r logits] <- a, gates[.., i logits] <- b,
+// y <- gelu_tanh(y)).  Pass 2, a thread a channel of a request: S <- a S + b along the rows in order, out = S * y.
+__global__ __launch_bounds__(256) void rglru_terms_kernel(RglruArgs p, int rows) {
+  const int c = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+  if (c >= p.channels || p.positions[row] < 0) return;
+  const int blk = c / p.bs, o = c % p.bs;
+  float* zr = const_cast<float*>(p.gates) + (size_t)row * p.ldg + (size_t)blk * 2 * p.bs + o;
+  float* yy = const_cast<float*>(p.y) + (size_t)row * p.ldy + c;
+  float a, b;
+  rglru_terms(zr[0], zr[p.bs], p.u[(size_t)row * p.ldu + c], p.ra_bias[c], p.ri_bias[c], p.decay[c], a, b);
+  zr[0] = a;
+  zr[p.bs] = b;
+  *yy = gm_gelu_tanh(*yy);
+}
+
 template <typename TO>
 __global__ __launch_bounds__(64) void rglru_scan_kernel(RglruArgs p) {
   const int c = blockIdx.x * 64 + threadIdx.x, seq = blockIdx.y;
   const int first = p.seq_rows[2 * seq], n = p.seq_rows[2 * seq + 1], slot = p.slots[seq];
   if (c >= p.channels || n <= 0 || slot < 0 || p.positions[first] < 0) return;
   const int blk = c / p.bs, o = c % p.bs;
-  const float br = p.ra_bias[c], bi = p.ri_bias[c], dc = p.decay[c];
-  const float* zr = p.gates + (size_t)first * p.ldg + (size_t)blk * 2 * p.bs + o;
-  const float* zi = zr + p.bs;
-  const float* u = p.u + (size_t)first * p.ldu + c;
+  const float* za = p.gates + (size_t)first * p.ldg + (size_t)blk * 2 * p.bs + o;
+  const float* zb = za + p.bs;
   const float* y = p.y + (size_t)first * p.ldy + c;
   TO* out = reinterpret_cast<TO*>(p.out) + (size_t)first * p.ldo + c;
   float* st = p.state + (size_t)slot * p.state_ld + c;
   float S = *st;
-  constexpr int UN = 4;
+  constexpr int UN = 16;
   int t = 0;
   for (; t + UN <= n; t += UN) {
-    float vzr[UN], vzi[UN], vu[UN], vy[UN];
+    float va[UN], vb[UN], vy[UN];
 #pragma unroll
     for (int j = 0; j < UN; ++j) {
-      vzr[j] = zr[(size_t)(t + j) * p.ldg];
-      vzi[j] = zi[(size_t)(t + j) * p.ldg];
-      vu[j] = u[(size_t)(t + j) * p.ldu];
+      va[j] = za[(size_t)(t + j) * p.ldg];
+      vb[j] = zb[(size_t)(t + j) * p.ldg];
       vy[j] = y[(size_t)(t + j) * p.ldy];
     }
 #pragma unroll
     for (int j = 0; j < UN; ++j) {
-      float a, b;
-      rglru_terms(vzr[j], vzi[j], vu[j], br, bi, dc, a, b);
-      S = fmaf(a, S, b);
-      gm_store(out + (size_t)(t + j) * p.ldo, S * gm_gelu_tanh(vy[j]));
+      S = fmaf(va[j], S, vb[j]);
+      gm_store(out + (size_t)(t + j) * p.ldo, S * vy[j]);
     }
   }
   for (; t < n; ++t) {
-    float a, b;
-    rglru_terms(zr[(size_t)t * p.ldg], zi[(size_t)t * p.ldg], u[(size_t)t * p.ldu], br, bi, dc, a, b);
-    S = fmaf(a, S, b);
-    gm_store(out + (size_t)t * p.ldo, S * gm_gelu_tanh(y[(size_t)t * p.ldy]));
+    S = fmaf(za[(size_t)t * p.ldg], S, zb[(size_t)t * p.ldg]);
+    gm_store(out + (size_t)t * p.ldo, S * y[(size_t)t * p.ldy]);
   }
   *st = S;
 }
 
-extern "C" int bw_rglru_scan(const float* y, int ldy, const float* u, int ldu, const float* gates, int ldg, const float* ra_bias,
+extern "C" int bw_rglru_scan(float* y, int ldy, const float* u, int ldu, float* gates, int ldg, const float* ra_bias,
                              const float* ri_bias, const float* decay, float* state, long long state_ld, void* out,
                              int out_is_bf16, int ldo, const int32_t* seq_rows, const int32_t* slots, const int32_t* positions,
-                             int nseq, int channels, int bs, void* stream) {
-  if (nseq <= 0 || channels <= 0) return 0;
-  if (bs <= 0 || channels % bs || nseq > 65535) return -2;
+                             int nseq, int rows, int channels, int bs, void* stream) {
+  if (nseq <= 0 || channels <= 0 || rows <= 0) return 0;
+  if (bs <= 0 || channels % bs || nseq > 65535 || rows > 65535) return -2;
   RglruArgs p{y, u, gates, ra_bias, ri_bias, decay, state, out, seq_rows, slots, positions, state_ld, ldy, ldu, ldg, ldo, channels, bs};
+  hipLaunchKernelGGL(rglru_terms_kernel, dim3((channels + 255) / 256, rows), dim3(256), 0, (hipStream_t)stream, p, rows);
   const dim3 grid((channels + 63) / 64, nseq);
   if (out_is_bf16) hipLaunchKernelGGL(rglru_scan_kernel<bf16_t>, grid, dim3(64), 0, (hipStream_t)stream, p);
   else hipLaunchKernelGGL(rglru_scan_kernel<float>, grid, dim3(64), 0, (hipStream_t)stream, p);
@@ -339,26 +349,62 @@ extern "C" int bw_rglru_scan(const float* y, int ldy, const float* u, int ldu, c
 
 // ------------------------------------------------------------------------------ x += rmsnorm(y) * w
 
+// A workgroup a row.  Thread t owns elements t, t + 256, ...; its sum of squares is one chain over them, the waves'
+// sums are joined by the butterflies of wave_sum and the four of them added in wave order: the same order for every
+// row of every launch.  rounded (optional): the new row once more, rounded to bfloat16, for the next sublayer's products.
 template <typename WT>
 __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__ y, int ldy, const WT* __restrict__ w, float* __restrict__ x,
-                                                       int ldx, int rows, int dim, float eps) {
-  const int row = blockIdx.x * 4 + wave_index(), lane = threadIdx.x & 63;
-  if (row >= rows) return;
+                                                       int ldx, bf16_t* __restrict__ rounded, int ldr, int dim, float eps) {
+  __shared__ float part[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
   const float* yr = y + (size_t)row * ldy;
+  constexpr int MAXV = 8;                       // rows of up to 256 * MAXV elements keep their values in registers
+  float v[MAXV];
   float acc = 0.0f;
-  for (int e = lane; e < dim; e += 64) acc = fmaf(yr[e], yr[e], acc);
+  if (dim <= 256 * MAXV) {
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+      const int e = tid + 256 * j;
+      v[j] = e < dim ? yr[e] : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) acc = fmaf(v[j], v[j], acc);
+  } else {
+    for (int e = tid; e < dim; e += 256) acc = fmaf(yr[e], yr[e], acc);
+  }
   acc = wave_sum(acc);
-  const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
+  if ((tid & 63) == 0) part[tid >> 6] = acc;
+  __syncthreads();
+  const float total = ((part[0] + part[1]) + part[2]) + part[3];
+  const float inv = 1.0f / sqrtf(total / (float)dim + eps);
   float* xr = x + (size_t)row * ldx;
-  for (int e = lane; e < dim; e += 64) xr[e] = xr[e] + (yr[e] * inv) * gm_load(w + e);
+  if (dim <= 256 * MAXV) {
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+      const int e = tid + 256 * j;
+      if (e < dim) {
+        const float nx = xr[e] + (v[j] * inv) * gm_load(w + e);
+        xr[e] = nx;
+        if (rounded != nullptr) rounded[(size_t)row * ldr + e] = f32_to_bf16(nx);
+      }
+    }
+  } else {
+    for (int e = tid; e < dim; e += 256) {
+      const float nx = xr[e] + (yr[e] * inv) * gm_load(w + e);
+      xr[e] = nx;
+      if (rounded != nullptr) rounded[(size_t)row * ldr + e] = f32_to_bf16(nx);
+    }
+  }
 }
 
-extern "C" int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, int rows, int dim, float eps,
-                           void* stream) {
+extern "C" int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, void* rounded, int ldr,
+                           int rows, int dim, float eps, void* stream) {
   if (rows <= 0) return 0;
-  const dim3 grid((rows + 3) / 4);
-  if (w_is_bf16) hipLaunchKernelGGL(norm_add_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const bf16_t*)w, x, ldx, rows, dim, eps);
-  else hipLaunchKernelGGL(norm_add_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const float*)w, x, ldx, rows, dim, eps);
+  const dim3 grid(rows);
+  if (w_is_bf16)
+    hipLaunchKernelGGL(norm_add_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const bf16_t*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps);
+  else
+    hipLaunchKernelGGL(norm_add_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const float*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps);
   return BW_LAUNCH_CHECK();
 }
 

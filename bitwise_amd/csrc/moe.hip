@@ -21,7 +21,7 @@
 #include "common.h"
 #include "api.h"
 
-#define MOE_TM 32            // slots a tile
+#define MOE_TM 64            // slots a tile
 #define MOE_MAX_EXPERTS 1024
 
 // ------------------------------------------------------------------------------ route
@@ -111,63 +111,63 @@ extern "C" int bw_moe_route(const float* logits, int ld, int rows, int experts, 
 
 // ------------------------------------------------------------------------------ plan
 
-// One workgroup.  sorted[p] = slot at sorted place p; place[slot] = p; tiles[t] = (expert, first place, slots, 0);
-// meta[0] = number of tiles.  Within an expert's run the slots ascend (every thread ranks its slots by counting the
-// equal experts before them), so the plan is the same from run to run.
-__global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ ids, int n, int E, int32_t* __restrict__ sorted,
+// One workgroup of 1024 threads.  sorted[p] = slot at sorted place p; place[slot] = p; tiles[t] = (expert, first place,
+// slots, 0); meta[0] = number of tiles.  Thread (expert e, segment g) walks segment g of the slots and counts those of
+// expert e; after a prefix over segments and experts it walks the segment again and hands out places.  Within an expert's
+// run the slots ascend, so the plan is the same from run to run.
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ ids, int n, int E, int segs, int32_t* __restrict__ sorted,
                                                         int32_t* __restrict__ place, int32_t* __restrict__ tiles,
-                                                        int32_t* __restrict__ meta, int32_t* __restrict__ rank) {
+                                                        int32_t* __restrict__ meta) {
+  __shared__ int seg_count[1024];       // [expert][segment]; after the prefix: slots of the expert in earlier segments
   __shared__ int counts[MOE_MAX_EXPERTS], start[MOE_MAX_EXPERTS], tile0[MOE_MAX_EXPERTS];
-  __shared__ int chunk_counts[MOE_MAX_EXPERTS];
   const int tid = threadIdx.x;
-  for (int e = tid; e < E; e += 1024) counts[e] = 0;
-  __syncthreads();
-  // the rank of a slot among the slots of its expert, in slot order: chunks of 1024 slots, one after the other
-  for (int base = 0; base < n; base += 1024) {
-    for (int e = tid; e < E; e += 1024) chunk_counts[e] = 0;
-    __syncthreads();
-    const int sidx = base + tid;
-    int e = -1;
-    if (sidx < n) e = ids[sidx];
-    // rank inside the chunk: ballot per wave would do; with few experts a count over the chunk's earlier slots through
-    // LDS atomics gives an order that changes from run to run, so the earlier slots are counted directly
-    __shared__ int chunk_ids[1024];
-    chunk_ids[tid] = e;
-    __syncthreads();
-    if (e >= 0) {
-      int before = 0;
-      for (int j = 0; j < tid; ++j) before += chunk_ids[j] == e;
-      rank[sidx] = counts[e] + before;
-      atomicAdd(&chunk_counts[e], 1);
-    }
-    __syncthreads();
-    for (int x = tid; x < E; x += 1024) counts[x] += chunk_counts[x];
-    __syncthreads();
+  const int e = tid / segs, g = tid % segs;
+  const int seg_len = (n + segs - 1) / segs;
+  const int s0 = g * seg_len, s1 = min(n, s0 + seg_len);
+  const bool mine = e < E;
+  if (mine) {
+    int c = 0;
+    for (int sidx = s0; sidx < s1; ++sidx) c += ids[sidx] == e;
+    seg_count[tid] = c;
   }
+  __syncthreads();
+  if (tid < E) {
+    int c = 0;
+    for (int k = 0; k < segs; ++k) {
+      const int v = seg_count[tid * segs + k];
+      seg_count[tid * segs + k] = c;
+      c += v;
+    }
+    counts[tid] = c;
+  }
+  __syncthreads();
   if (tid == 0) {
-    int s0 = 0, t0 = 0;
-    for (int e = 0; e < E; ++e) {
-      start[e] = s0;
-      tile0[e] = t0;
-      s0 += counts[e];
-      t0 += (counts[e] + MOE_TM - 1) / MOE_TM;
+    int p = 0, t = 0;
+    for (int x = 0; x < E; ++x) {
+      start[x] = p;
+      tile0[x] = t;
+      p += counts[x];
+      t += (counts[x] + MOE_TM - 1) / MOE_TM;
     }
-    meta[0] = t0;
+    meta[0] = t;
   }
   __syncthreads();
-  for (int sidx = tid; sidx < n; sidx += 1024) {
-    const int e = ids[sidx];
-    const int p = start[e] + rank[sidx];
-    sorted[p] = sidx;
-    place[sidx] = p;
+  if (mine) {
+    int p = start[e] + seg_count[tid];
+    for (int sidx = s0; sidx < s1; ++sidx)
+      if (ids[sidx] == e) {
+        sorted[p] = sidx;
+        place[sidx] = p;
+        ++p;
+      }
   }
-  for (int e = tid; e < E; e += 1024) {
-    const int nt = (counts[e] + MOE_TM - 1) / MOE_TM;
+  for (int x = tid; x < E; x += 1024) {
+    const int nt = (counts[x] + MOE_TM - 1) / MOE_TM;
     for (int t = 0; t < nt; ++t) {
-      int32_t* rec = tiles + (size_t)(tile0[e] + t) * 4;
-      rec[0] = e;
-      rec[1] = start[e] + t * MOE_TM;
-      rec[2] = min(MOE_TM, counts[e] - t * MOE_TM);
+      int32_t* rec = tiles + (size_t)(tile0[x] + t) * 4;
+      rec[0] = x;
+      rec[1] = start[x] + t * MOE_TM;
+      rec[2] = min(MOE_TM, counts[x] - t * MOE_TM);
       rec[3] = 0;
     }
   }
@@ -179,10 +179,12 @@ extern "C" int bw_moe_max_tiles(int slots, int experts) {
 }
 
 extern "C" int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* sorted, int32_t* place, int32_t* tiles,
-                           int32_t* meta, int32_t* rank, void* stream) {
+                           int32_t* meta, void* stream) {
   if (slots <= 0) return 0;
   if (experts < 1 || experts > MOE_MAX_EXPERTS) return -2;
-  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ids, slots, experts, sorted, place, tiles, meta, rank);
+  int segs = 1;
+  while (segs * 2 * experts <= 1024) segs *= 2;
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ids, slots, experts, segs, sorted, place, tiles, meta);
   return BW_LAUNCH_CHECK();
 }
 
@@ -205,27 +207,29 @@ struct MoeArgs {
 };
 
 // A workgroup of four waves per (tile of MOE_TM slots, 128 output columns); a wave owns 32 columns, for GATE_UP of
-// the gate and of the up matrix both.  Operands go from memory straight into registers: lane (r, g) holds row r's
-// (or column r's) elements k + 8g .. k + 8g + 7.  Rows of a tile past its slots read row 0 of x and are never stored.
+// the gate and of the up matrix both, and all of the tile's rows.  Operands go from memory straight into registers: lane
+// (r, g) holds row r's (or column r's) elements k + 8g .. k + 8g + 7; three sets of operand registers keep two steps of
+// the inner size in flight behind the one being multiplied.  Blocks of 16 rows past the tile's slots are skipped (a scalar
+// branch: the matrix cores ignore the execution mask); rows past them inside a block read the tile's first row and are
+// never stored.
 template <bool GATE_UP>
 __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w,
                                                        void* __restrict__ out, int ldo) {
-  const int tile = blockIdx.y;
+  const int tile = blockIdx.x;
   if (tile >= a.meta[0]) return;
   const int wave = wave_index(), lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
-  const int e = a.tiles[tile * 4], p0 = a.tiles[tile * 4 + 1], cnt = a.tiles[tile * 4 + 2];
-  const int n0 = blockIdx.x * 128 + wave * 32;
+  const int e = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4]), p0 = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4 + 1]),
+            cnt = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4 + 2]);
+  const int n0 = blockIdx.y * 128 + wave * 32;
   if (n0 >= a.N) return;                                   // (scalar: the wave's columns lie past the matrix)
   constexpr int NB = GATE_UP ? 4 : 2, MB = MOE_TM / 16;
+  const int mb_live = (cnt + 15) >> 4;                     // blocks of 16 rows that hold a slot
   const bf16_t* xr[MB];
 #pragma unroll
   for (int i = 0; i < MB; ++i) {
     const int q = 16 * i + r;
-    size_t src_row = 0;
-    if (q < cnt) src_row = GATE_UP ? (size_t)(a.sorted[p0 + q] / a.top) : (size_t)(p0 + q);
-    else if (!GATE_UP) src_row = (size_t)p0;
-    else src_row = (size_t)(a.sorted[p0] / a.top);
-    xr[i] = x + src_row * ldx + 8 * g;
+    const int pq = p0 + (q < cnt ? q : 0);
+    xr[i] = x + (GATE_UP ? (size_t)(a.sorted[pq] / a.top) : (size_t)pq) * ldx + 8 * g;
   }
   // weights of expert e: GATE_UP [2N, K] (gate rows, then up rows), else [N, K]
   const bf16_t* wr[NB];
@@ -243,29 +247,37 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* 
     for (int b = 0; b < NB; ++b) acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const u32x4 zero = {0u, 0u, 0u, 0u};
   const int K = a.K;
-  auto load = [&](int k, u32x4 (&af)[MB], u32x4 (&bfr)[NB]) {
-    const bool live = k + 8 * g + 8 <= K;                  // (K is a multiple of 8)
+  struct Ops { u32x4 af[MB], bfr[NB]; };
+  auto load = [&](int k, Ops& o) {
+    const bool live = k + 8 * g + 8 <= K;                  // (K is a multiple of 8; past K nothing is asked of memory)
 #pragma unroll
-    for (int i = 0; i < MB; ++i) af[i] = live ? *reinterpret_cast<const u32x4*>(xr[i] + k) : zero;
+    for (int i = 0; i < MB; ++i) o.af[i] = (live && i < mb_live) ? *reinterpret_cast<const u32x4*>(xr[i] + k) : zero;
 #pragma unroll
-    for (int b = 0; b < NB; ++b) bfr[b] = live ? *reinterpret_cast<const u32x4*>(wr[b] + k) : zero;
+    for (int b = 0; b < NB; ++b) o.bfr[b] = live ? *reinterpret_cast<const u32x4*>(wr[b] + k) : zero;
   };
-  u32x4 a0[MB], b0[NB], a1[MB], b1[NB];
-  load(0, a0, b0);
-  for (int k = 0; k < K; k += 64) {
-    if (k + 32 < K) load(k + 32, a1, b1);
+  auto mma = [&](const Ops& o) {
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
-#pragma unroll
-      for (int b = 0; b < NB; ++b)
-        acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a0[i]), as_bf16x8(b0[b]), acc[i][b], 0, 0, 0);
-    if (k + 32 < K) {                                       // (scalar)
-      if (k + 64 < K) load(k + 64, a0, b0);
-#pragma unroll
-      for (int i = 0; i < MB; ++i)
+    for (int i = 0; i < MB; ++i) {
+      if (i < mb_live) {                                   // scalar
 #pragma unroll
         for (int b = 0; b < NB; ++b)
-          acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a1[i]), as_bf16x8(b1[b]), acc[i][b], 0, 0, 0);
+          acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(o.af[i]), as_bf16x8(o.bfr[b]), acc[i][b], 0, 0, 0);
+      }
+    }
+  };
+  Ops o0, o1, o2;
+  load(0, o0);
+  load(32, o1);
+  for (int k = 0; k < K; k += 96) {
+    load(k + 64, o2);
+    mma(o0);
+    if (k + 32 < K) {                                      // (scalar)
+      load(k + 96, o0);
+      mma(o1);
+    }
+    if (k + 64 < K) {
+      load(k + 128, o1);
+      mma(o2);
     }
   }
   // accumulator element q of block (i, b): slot 16 i + 4 g + q, column 16 b' + r
@@ -275,19 +287,14 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* 
     for (int q = 0; q < 4; ++q) {
       const int m = 16 * i + 4 * g + q;
       if (m >= cnt) continue;
-      if constexpr (GATE_UP) {
 #pragma unroll
-        for (int cb = 0; cb < 2; ++cb) {
-          const int n = n0 + 16 * cb + r;
-          if (n < a.N)
-            reinterpret_cast<bf16_t*>(out)[(size_t)(p0 + m) * ldo + n] = f32_to_bf16(moe_act(acc[i][cb][q], acc[i][2 + cb][q], a.limit, a.alpha));
-        }
-      } else {
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb) {
-          const int n = n0 + 16 * cb + r;
-          if (n < a.N) reinterpret_cast<float*>(out)[(size_t)(p0 + m) * ldo + n] = acc[i][cb][q];
-        }
+      for (int cb = 0; cb < 2; ++cb) {
+        const int n = n0 + 16 * cb + r;
+        if (n >= a.N) continue;
+        if constexpr (GATE_UP)
+          reinterpret_cast<bf16_t*>(out)[(size_t)(p0 + m) * ldo + n] = f32_to_bf16(moe_act(acc[i][cb][q], acc[i][2 + cb][q], a.limit, a.alpha));
+        else
+          reinterpret_cast<float*>(out)[(size_t)(p0 + m) * ldo + n] = acc[i][cb][q];
       }
     }
 }
@@ -300,10 +307,10 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* 
 template <bool GATE_UP, typename WT>
 __global__ __launch_bounds__(64) void moe_f32_kernel(MoeArgs a, const float* __restrict__ x, int ldx, const WT* __restrict__ w,
                                                      float* __restrict__ out, int ldo, int round_out) {
-  const int tile = blockIdx.y;
+  const int tile = blockIdx.x;
   if (tile >= a.meta[0]) return;
   const int e = a.tiles[tile * 4], p0 = a.tiles[tile * 4 + 1], cnt = a.tiles[tile * 4 + 2];
-  const int n = blockIdx.x * 64 + threadIdx.x;
+  const int n = blockIdx.y * 64 + threadIdx.x;
   if (n >= a.N) return;
   const size_t wbase = (size_t)e * (GATE_UP ? 2 : 1) * a.N * a.K;
   const WT* wg = w + wbase + (size_t)n * a.K;
@@ -331,17 +338,17 @@ extern "C" int bw_moe_experts(const void* x, int x_is_bf16, int ldx, const void*
                               const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int max_tiles, int top, int K,
                               int N, int gate_up, float limit, float alpha, int round_out, void* stream) {
   if (max_tiles <= 0) return 0;
-  if (max_tiles > 65535 || K <= 0 || N <= 0) return -2;
+  if (K <= 0 || N <= 0 || (N + 63) / 64 > 65535) return -2;
   MoeArgs a{sorted, tiles, meta, top, K, N, limit, alpha};
   hipStream_t s = (hipStream_t)stream;
   if (x_is_bf16) {
     if (!w_is_bf16 || K % 8 || ldx % 8) return -3;
-    const dim3 grid((N + 127) / 128, max_tiles);
+    const dim3 grid(max_tiles, (N + 127) / 128);
     if (gate_up) hipLaunchKernelGGL(moe_mfma_kernel<true>, grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
     else hipLaunchKernelGGL(moe_mfma_kernel<false>, grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
     return BW_LAUNCH_CHECK();
   }
-  const dim3 grid((N + 63) / 64, max_tiles);
+  const dim3 grid(max_tiles, (N + 63) / 64);
   if (gate_up) {
     if (w_is_bf16) hipLaunchKernelGGL((moe_f32_kernel<true, bf16_t>), grid, dim3(64), 0, s, a, (const float*)x, ldx, (const bf16_t*)w, (float*)out, ldo, round_out);
     else hipLaunchKernelGGL((moe_f32_kernel<true, float>), grid, dim3(64), 0, s, a, (const float*)x, ldx, (const float*)w, (float*)out, ldo, round_out);

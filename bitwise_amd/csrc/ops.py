@@ -99,12 +99,12 @@ _SIGS = {
                           c_int, c_void_p],
     "bw_gate_mul": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_rglru_scan": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
-                      c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
-    "bw_norm_add": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+                      c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_norm_add": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "bw_softcap": [c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "bw_moe_route": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "bw_moe_max_tiles": [c_int, c_int],
-    "bw_moe_plan": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "bw_moe_plan": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_moe_experts": [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
                        c_int, c_int, c_int, c_float, c_float, c_int, c_void_p],
     "bw_moe_combine": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
@@ -1031,11 +1031,13 @@ def gate_mul(av: torch.Tensor, head_size: int, g: torch.Tensor, out: torch.Tenso
 
 def rglru_scan(y: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, ra_bias: torch.Tensor, ri_bias: torch.Tensor,
                decay: torch.Tensor, state: torch.Tensor, out: torch.Tensor, seq_rows: torch.Tensor, slots: torch.Tensor,
-               positions: torch.Tensor, nseq: int, channels: int, block: int) -> None:
+               positions: torch.Tensor, nseq: int, rows: int, channels: int, block: int) -> None:
     """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) * i_t * u_t per channel along every request's rows, from and to ``state``
     [slots, >= channels]; a_t = exp(decay * r_t), r_t = sigmoid(gate logits + ra_bias), i_t likewise with ri_bias;
     ``gates`` [rows, channels/block * 2*block]: per block its recurrence-gate logits, then its input-gate logits;
-    out = S_t * gelu_tanh(y_t).  y, u: float32 with contiguous rows (column slices will do)."""
+    out = S_t * gelu_tanh(y_t).  y, u: float32 with contiguous rows (column slices will do).  Two launches: what a row
+    contributes by itself (factor, addend, activation) for all ``rows`` rows at once, written over ``gates`` and ``y``,
+    then the walk along each request's rows."""
     for t, what in ((y, "y"), (u, "u"), (gates, "gates"), (state, "state")):
         if t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or not t.is_cuda:
             raise ValueError(f"rglru_scan: {what} must be a float32 GPU matrix with contiguous rows")
@@ -1047,22 +1049,29 @@ def rglru_scan(y: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, ra_bias: t
         _need(t, torch.int32, what)
     if channels % block or min(y.shape[1], u.shape[1], state.shape[1]) < channels or gates.shape[1] < 2 * channels or out.shape[1] != channels:
         raise ValueError("rglru_scan: widths do not fit the channels")
-    if seq_rows.numel() < 2 * nseq or slots.numel() < nseq:
-        raise ValueError("rglru_scan: fewer request records than requests")
+    if seq_rows.numel() < 2 * nseq or slots.numel() < nseq or positions.numel() < rows or min(y.shape[0], u.shape[0], gates.shape[0], out.shape[0]) < rows:
+        raise ValueError("rglru_scan: fewer request records than requests, or buffers shorter than the rows")
     _check(_fn("bw_rglru_scan")(y.data_ptr(), y.stride(0), u.data_ptr(), u.stride(0), gates.data_ptr(), gates.stride(0),
                                 ra_bias.data_ptr(), ri_bias.data_ptr(), decay.data_ptr(), state.data_ptr(), state.stride(0),
                                 out.data_ptr(), _act_out(out, "out"), out.stride(0), seq_rows.data_ptr(), slots.data_ptr(),
-                                positions.data_ptr(), int(nseq), channels, block, _stream()), "rglru_scan")
+                                positions.data_ptr(), int(nseq), int(rows), channels, block, _stream()), "rglru_scan")
 
 
-def norm_add(y: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, rows: int, eps: float) -> None:
-    """x[:rows] += y / sqrt(mean(y^2) + eps) * weight, all 32-bit."""
+def norm_add(y: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, rows: int, eps: float,
+             rounded: Optional[torch.Tensor] = None) -> None:
+    """x[:rows] += y / sqrt(mean(y^2) + eps) * weight, all 32-bit.  ``rounded`` (bfloat16, x's shape): also receives the new
+    rows rounded, for products that follow."""
     _need(y, torch.float32, "y")
     _need(x, torch.float32, "x")
     dim = x.shape[1]
     if y.shape[1] != dim or weight.numel() != dim or not weight.is_cuda or min(x.shape[0], y.shape[0]) < rows:
         raise ValueError("norm_add: y, weight and x do not fit")
+    if rounded is not None:
+        _need(rounded, torch.bfloat16, "rounded")
+        if rounded.shape[1] != dim or rounded.shape[0] < rows:
+            raise ValueError("norm_add: the rounded copy does not fit")
     _check(_fn("bw_norm_add")(y.data_ptr(), y.stride(0), weight.data_ptr(), _is_bf16(weight, "weight"), x.data_ptr(), x.stride(0),
+                              0 if rounded is None else rounded.data_ptr(), 0 if rounded is None else rounded.stride(0),
                               rows, dim, float(eps), _stream()), "norm_add")
 
 
@@ -1098,14 +1107,14 @@ def moe_route(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int,
 
 
 def moe_plan(ids: torch.Tensor, slots: int, experts: int, sorted_slots: torch.Tensor, place: torch.Tensor, tiles: torch.Tensor,
-             meta: torch.Tensor, rank: torch.Tensor) -> None:
+             meta: torch.Tensor) -> None:
     """The (row, choice) pairs sorted by expert and cut into tiles of one expert each (see moe.hip)."""
-    for t, what in ((ids, "ids"), (sorted_slots, "sorted"), (place, "place"), (tiles, "tiles"), (meta, "meta"), (rank, "rank")):
+    for t, what in ((ids, "ids"), (sorted_slots, "sorted"), (place, "place"), (tiles, "tiles"), (meta, "meta")):
         _need(t, torch.int32, what)
-    if min(ids.numel(), sorted_slots.numel(), place.numel(), rank.numel()) < slots or tiles.numel() < 4 * moe_max_tiles(slots, experts) or meta.numel() < 1:
+    if min(ids.numel(), sorted_slots.numel(), place.numel()) < slots or tiles.numel() < 4 * moe_max_tiles(slots, experts) or meta.numel() < 1:
         raise ValueError("moe_plan: buffers too small")
     _check(_fn("bw_moe_plan")(ids.data_ptr(), slots, experts, sorted_slots.data_ptr(), place.data_ptr(), tiles.data_ptr(),
-                              meta.data_ptr(), rank.data_ptr(), _stream()), "moe_plan")
+                              meta.data_ptr(), _stream()), "moe_plan")
 
 
 def moe_experts(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_slots: torch.Tensor, tiles: torch.Tensor,

@@ -162,6 +162,7 @@ class AssembledModel:
         if len(ctx.calls) != len(self.calls):
             raise ValueError("the step context carries no bindings for this model's layer calls")
         ws = ctx.ws
+        ctx.forward_notes = {}           # what parts tell later parts within this pass (a rounded copy of the stream that is current)
         x = self.embedding.forward(ctx)
         for call in ctx.calls:
             self.layers[call.layer].forward(ctx, call, x)

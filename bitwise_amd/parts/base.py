@@ -173,8 +173,9 @@ class Norm(Part):
         """x: [rows, width] 32-bit residual stream -> normed rows in the activation dtype."""
         raise NotImplementedError
 
-    def add_normed(self, ctx, y, x) -> None:
-        """x += norm(y), both 32-bit [rows, width]: the norm of a sublayer's output on its way into the residual stream."""
+    def add_normed(self, ctx, y, x, rounded=None) -> None:
+        """x += norm(y), both 32-bit [rows, width]: the norm of a sublayer's output on its way into the residual stream.
+        ``rounded`` (bfloat16 [rows, width]), if given, also receives the new x rounded."""
         raise NotImplementedError
 
 

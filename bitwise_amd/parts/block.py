@@ -74,16 +74,29 @@ class PostNormBlock(Block):
             raise ValueError("postnorm block: a feed-forward and its norm come together or not at all")
 
     def _input(self, ctx, x):
+        """The stream as the sublayer's products take it.  The kernel that adds a sublayer's normed output into the stream
+        leaves the rounded copy behind (``forward_notes``: what parts tell later parts within one forward pass), so only
+        a model's first layer converts."""
         if not self.rt.bf16:
             return x
         h = ctx.ws.buffer("stream_rounded", x.shape[1], torch.bfloat16)
-        ops.convert(x, h, ctx.rows)
+        notes = getattr(ctx, "forward_notes", None)
+        if notes is None or notes.get("stream_rounded") is not x:
+            ops.convert(x, h, ctx.rows)
         return h
+
+    def _add(self, ctx, norm, y, x) -> None:
+        notes = getattr(ctx, "forward_notes", None)
+        if self.rt.bf16 and notes is not None:
+            norm.add_normed(ctx, y, x, rounded=ctx.ws.buffer("stream_rounded", x.shape[1], torch.bfloat16))
+            notes["stream_rounded"] = x
+        else:
+            norm.add_normed(ctx, y, x)
 
     def forward(self, ctx, call, x) -> None:
         y = ctx.ws.buffer("sublayer_out", x.shape[1], torch.float32)
         self.mixer.forward_out(ctx, call, self._input(ctx, x), y)
-        self.mixer_norm.add_normed(ctx, y, x)
+        self._add(ctx, self.mixer_norm, y, x)
         if self.feed_forward is not None:
             self.feed_forward.forward_out(ctx, self._input(ctx, x), y)
-            self.ffn_norm.add_normed(ctx, y, x)
+            self._add(ctx, self.ffn_norm, y, x)

@@ -55,8 +55,9 @@ class RoutedExperts(FeedForward):
 
     def bind(self, tensors) -> None:
         dev = self.rt.device
-        # the router's product stays 32-bit in either mode
-        self.router = Linear(tensors["router"], self.rt, matrix_cores=False)
+        # the router's sums are 32-bit in either mode; in bfloat16 mode the rows arrive rounded and the weights are stored
+        # so, their products are exact in 32 bits and the matrix cores add them up in 32 bits
+        self.router = Linear(tensors["router"], self.rt)
         kinds = {tensors[f"e{j}.{n}"].dtype for j in range(self.experts) for n in ("gate", "up", "down")}
         if len(kinds) != 1:
             raise ValueError("the experts of one feed-forward must be stored in one dtype to be stacked")
@@ -87,10 +88,9 @@ class RoutedExperts(FeedForward):
         ops.moe_route(logits, rows, self.top, self.groups, self.keep, ids, wts)
         sorted_slots = ws.buffer("moe_sorted", most, torch.int32, rows=1)
         place = ws.buffer("moe_place", most, torch.int32, rows=1)
-        rank = ws.buffer("moe_rank", most, torch.int32, rows=1)
         tiles = ws.buffer("moe_tiles", 4 * ops.moe_max_tiles(most, self.experts), torch.int32, rows=1)
         meta = ws.buffer("moe_meta", 4, torch.int32, rows=1)
-        ops.moe_plan(ids, slots, self.experts, sorted_slots, place, tiles, meta, rank)
+        ops.moe_plan(ids, slots, self.experts, sorted_slots, place, tiles, meta)
         if self.mfma:
             x, act_dtype = h, torch.bfloat16
         else:

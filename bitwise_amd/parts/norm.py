@@ -49,9 +49,9 @@ class RMSNorm(Norm):
         ops.rmsnorm(x, self.weight, out, rows, self.eps)
         return out
 
-    def add_normed(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
-        """x += y / sqrt(mean(y^2) + eps) * weight, one kernel, all 32-bit."""
-        ops.norm_add(y, self.weight, x, ctx.rows, self.eps)
+    def add_normed(self, ctx, y: torch.Tensor, x: torch.Tensor, rounded: Optional[torch.Tensor] = None) -> None:
+        """x += y / sqrt(mean(y^2) + eps) * weight, one kernel, all 32-bit; ``rounded``: the new x once more, in bfloat16."""
+        ops.norm_add(y, self.weight, x, ctx.rows, self.eps, rounded)
 
 
 @register_norm("rmsnorm_shift")

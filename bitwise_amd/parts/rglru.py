@@ -93,7 +93,7 @@ class RealGatedLRU(Mixer):
         ops.headwise_linear(u, 0, self.bs, self.gate_w, gates, 0, 2 * self.bs, rows)
         act = ws.buffer("rglru_out", R, self.rt.act_dtype)
         ops.rglru_scan(proj, u, gates, self.ra_b, self.ri_b, self.decay, call.state[:, (self.taps - 1) * R:], act,
-                       ctx.seq_rows, ctx.slots, ctx.positions, ctx.nseq, R, self.bs)
+                       ctx.seq_rows, ctx.slots, ctx.positions, ctx.nseq, rows, R, self.bs)
         if add:
             self.o.add_into(ws, act, target, rows)
         else:
