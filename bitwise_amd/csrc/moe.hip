@@ -21,7 +21,8 @@
 #include "common.h"
 #include "api.h"
 
-#define MOE_TM 64            // slots a tile
+#define MOE_TM 64            // slots a tile of a step with many slots
+#define MOE_SMALL_SLOTS 1024  // steps of up to this many slots get tiles of 16
 #define MOE_MAX_EXPERTS 1024
 
 // ------------------------------------------------------------------------------ route
@@ -112,23 +113,30 @@ extern "C" int bw_moe_route(const float* logits, int ld, int rows, int experts, 
 // ------------------------------------------------------------------------------ plan
 
 // One workgroup of 1024 threads.  sorted[p] = slot at sorted place p; place[slot] = p; tiles[t] = (expert, first place,
-// slots, 0); meta[0] = number of tiles.  Thread (expert e, segment g) walks segment g of the slots and counts those of
-// expert e; after a prefix over segments and experts it walks the segment again and hands out places.  Within an expert's
-// run the slots ascend, so the plan is the same from run to run.
-__global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ ids, int n, int E, int segs, int32_t* __restrict__ sorted,
-                                                        int32_t* __restrict__ place, int32_t* __restrict__ tiles,
-                                                        int32_t* __restrict__ meta) {
+// slots, 0) with up to tm slots a tile; meta[0] = number of tiles.  Thread (segment g, expert e) walks segment g of the
+// slots (from LDS, where the workgroup has put them if they fit) and counts those of expert e; after a prefix over
+// segments and experts it walks the segment again and hands out places.  Within an expert's run the slots ascend, so
+// the plan is the same from run to run.
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ ids, int n, int E, int segs, int tm, int staged,
+                                                        int32_t* __restrict__ sorted, int32_t* __restrict__ place,
+                                                        int32_t* __restrict__ tiles, int32_t* __restrict__ meta) {
+  extern __shared__ int plan_ids[];     // [n] if staged
   __shared__ int seg_count[1024];       // [expert][segment]; after the prefix: slots of the expert in earlier segments
   __shared__ int counts[MOE_MAX_EXPERTS], start[MOE_MAX_EXPERTS], tile0[MOE_MAX_EXPERTS];
   const int tid = threadIdx.x;
-  const int e = tid / segs, g = tid % segs;
+  if (staged) {
+    for (int sidx = tid; sidx < n; sidx += 1024) plan_ids[sidx] = ids[sidx];
+    __syncthreads();
+  }
+  const int* src = staged ? plan_ids : ids;
+  const int e = tid % E, g = tid / E;
   const int seg_len = (n + segs - 1) / segs;
   const int s0 = g * seg_len, s1 = min(n, s0 + seg_len);
-  const bool mine = e < E;
+  const bool mine = g < segs;
   if (mine) {
     int c = 0;
-    for (int sidx = s0; sidx < s1; ++sidx) c += ids[sidx] == e;
-    seg_count[tid] = c;
+    for (int sidx = s0; sidx < s1; ++sidx) c += src[sidx] == e;
+    seg_count[e * segs + g] = c;
   }
   __syncthreads();
   if (tid < E) {
@@ -147,34 +155,38 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restric
       start[x] = p;
       tile0[x] = t;
       p += counts[x];
-      t += (counts[x] + MOE_TM - 1) / MOE_TM;
+      t += (counts[x] + tm - 1) / tm;
     }
     meta[0] = t;
   }
   __syncthreads();
   if (mine) {
-    int p = start[e] + seg_count[tid];
+    int p = start[e] + seg_count[e * segs + g];
     for (int sidx = s0; sidx < s1; ++sidx)
-      if (ids[sidx] == e) {
+      if (src[sidx] == e) {
         sorted[p] = sidx;
         place[sidx] = p;
         ++p;
       }
   }
   for (int x = tid; x < E; x += 1024) {
-    const int nt = (counts[x] + MOE_TM - 1) / MOE_TM;
+    const int nt = (counts[x] + tm - 1) / tm;
     for (int t = 0; t < nt; ++t) {
       int32_t* rec = tiles + (size_t)(tile0[x] + t) * 4;
       rec[0] = x;
-      rec[1] = start[x] + t * MOE_TM;
-      rec[2] = min(MOE_TM, counts[x] - t * MOE_TM);
+      rec[1] = start[x] + t * tm;
+      rec[2] = min(tm, counts[x] - t * tm);
       rec[3] = 0;
     }
   }
 }
 
+// Slots a tile: few slots a step (decoded tokens) get tiles of 16, whose kernel keeps many steps of weights in flight;
+// prompt portions get tiles of 64, whose kernel reuses every weight it loads for four blocks of rows.
+extern "C" int bw_moe_tile_rows(int slots) { return slots <= MOE_SMALL_SLOTS ? 16 : MOE_TM; }
+
 extern "C" int bw_moe_max_tiles(int slots, int experts) {
-  const int full = slots / MOE_TM;
+  const int full = slots / bw_moe_tile_rows(slots);
   return full + (experts < slots ? experts : slots);
 }
 
@@ -182,9 +194,10 @@ extern "C" int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* 
                            int32_t* meta, void* stream) {
   if (slots <= 0) return 0;
   if (experts < 1 || experts > MOE_MAX_EXPERTS) return -2;
-  int segs = 1;
-  while (segs * 2 * experts <= 1024) segs *= 2;
-  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ids, slots, experts, segs, sorted, place, tiles, meta);
+  const int segs = 1024 / experts;
+  const int staged = slots <= 12 * 1024;
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), staged ? (size_t)slots * sizeof(int) : 0, (hipStream_t)stream, ids, slots,
+                     experts, segs, bw_moe_tile_rows(slots), staged, sorted, place, tiles, meta);
   return BW_LAUNCH_CHECK();
 }
 
@@ -208,11 +221,12 @@ struct MoeArgs {
 
 // A workgroup of four waves per (tile of MOE_TM slots, 128 output columns); a wave owns 32 columns, for GATE_UP of
 // the gate and of the up matrix both, and all of the tile's rows.  Operands go from memory straight into registers: lane
-// (r, g) holds row r's (or column r's) elements k + 8g .. k + 8g + 7; three sets of operand registers keep two steps of
-// the inner size in flight behind the one being multiplied.  Blocks of 16 rows past the tile's slots are skipped (a scalar
+// (r, g) holds row r's (or column r's) elements k + 8g .. k + 8g + 7; a ring of DEPTH sets of operand registers keeps as
+// many steps of the inner size in flight.  MB blocks of 16 rows a tile: 4 for prompt portions, 1 with a deep ring for the
+// few rows of decoded tokens, where the weights stream from memory once and nothing is reused.  Blocks of 16 rows past the tile's slots are skipped (a scalar
 // branch: the matrix cores ignore the execution mask); rows past them inside a block read the tile's first row and are
 // never stored.
-template <bool GATE_UP>
+template <bool GATE_UP, int MB, int DEPTH>
 __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w,
                                                        void* __restrict__ out, int ldo) {
   const int tile = blockIdx.x;
@@ -222,7 +236,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* 
             cnt = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4 + 2]);
   const int n0 = blockIdx.y * 128 + wave * 32;
   if (n0 >= a.N) return;                                   // (scalar: the wave's columns lie past the matrix)
-  constexpr int NB = GATE_UP ? 4 : 2, MB = MOE_TM / 16;
+  constexpr int NB = GATE_UP ? 4 : 2;
   const int mb_live = (cnt + 15) >> 4;                     // blocks of 16 rows that hold a slot
   const bf16_t* xr[MB];
 #pragma unroll
@@ -265,19 +279,16 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* 
       }
     }
   };
-  Ops o0, o1, o2;
-  load(0, o0);
-  load(32, o1);
-  for (int k = 0; k < K; k += 96) {
-    load(k + 64, o2);
-    mma(o0);
-    if (k + 32 < K) {                                      // (scalar)
-      load(k + 96, o0);
-      mma(o1);
-    }
-    if (k + 64 < K) {
-      load(k + 128, o1);
-      mma(o2);
+  Ops ring[DEPTH];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load(32 * d, ring[d]);
+  for (int k = 0; k < K; k += 32 * DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (k + 32 * d < K) {                                // (scalar)
+        mma(ring[d]);
+        load(k + 32 * (d + DEPTH), ring[d]);
+      }
     }
   }
   // accumulator element q of block (i, b): slot 16 i + 4 g + q, column 16 b' + r
@@ -335,17 +346,23 @@ __global__ __launch_bounds__(64) void moe_f32_kernel(MoeArgs a, const float* __r
 }
 
 extern "C" int bw_moe_experts(const void* x, int x_is_bf16, int ldx, const void* w, int w_is_bf16, void* out, int ldo,
-                              const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int max_tiles, int top, int K,
-                              int N, int gate_up, float limit, float alpha, int round_out, void* stream) {
-  if (max_tiles <= 0) return 0;
+                              const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int slots, int max_tiles, int top,
+                              int K, int N, int gate_up, float limit, float alpha, int round_out, void* stream) {
+  const int tile_rows = bw_moe_tile_rows(slots);          // (as the plan was made)
+  if (max_tiles <= 0 || slots <= 0) return 0;
   if (K <= 0 || N <= 0 || (N + 63) / 64 > 65535) return -2;
   MoeArgs a{sorted, tiles, meta, top, K, N, limit, alpha};
   hipStream_t s = (hipStream_t)stream;
   if (x_is_bf16) {
     if (!w_is_bf16 || K % 8 || ldx % 8) return -3;
     const dim3 grid(max_tiles, (N + 127) / 128);
-    if (gate_up) hipLaunchKernelGGL(moe_mfma_kernel<true>, grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
-    else hipLaunchKernelGGL(moe_mfma_kernel<false>, grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+    if (tile_rows == 16) {
+      if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, 1, 8>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+      else hipLaunchKernelGGL((moe_mfma_kernel<false, 1, 12>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+    } else {
+      if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, MOE_TM / 16, 3>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+      else hipLaunchKernelGGL((moe_mfma_kernel<false, MOE_TM / 16, 3>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+    }
     return BW_LAUNCH_CHECK();
   }
   const dim3 grid(max_tiles, (N + 63) / 64);

@@ -88,7 +88,8 @@ class RoutedExperts(FeedForward):
         ops.moe_route(logits, rows, self.top, self.groups, self.keep, ids, wts)
         sorted_slots = ws.buffer("moe_sorted", most, torch.int32, rows=1)
         place = ws.buffer("moe_place", most, torch.int32, rows=1)
-        tiles = ws.buffer("moe_tiles", 4 * ops.moe_max_tiles(most, self.experts), torch.int32, rows=1)
+        # (room for the plan of any step: tiles hold 16 slots or more, and every expert may end with a partly filled one)
+        tiles = ws.buffer("moe_tiles", 4 * (most // 16 + self.experts), torch.int32, rows=1)
         meta = ws.buffer("moe_meta", 4, torch.int32, rows=1)
         ops.moe_plan(ids, slots, self.experts, sorted_slots, place, tiles, meta)
         if self.mfma:
