@@ -151,7 +151,7 @@ int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, in
 int bw_moe_max_tiles(int slots, int experts);
 int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* sorted, int32_t* place, int32_t* tiles,
                 int32_t* meta, void* stream);
-int bw_moe_experts(const void* x, int x_is_bf16, int ldx, const void* w, int w_is_bf16, void* out, int ldo,
+int bw_moe_experts(const void* x, int x_is_bf16, int ldx, int x_rows, const void* w, int w_is_bf16, void* out, int ldo,
                    const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int slots, int max_tiles, int top,
                    int K, int N, int gate_up, float limit, float alpha, int round_out, void* stream);
 int bw_moe_tile_rows(int slots);

@@ -13,7 +13,7 @@
 //   combine:  out[row] = sum over the row's choices, in the order they were chosen, of weight * its expert's output
 //
 // bfloat16 mode runs the two products on the matrix cores (v_mfma_f32_16x16x32_bf16 over the inner size ascending from
-// zero, one accumulator per 16 x 16 block of outputs): what a row gets depends on the row and its expert alone, not on
+// zero in steps of 64 elements, two instructions a step, one accumulator per 16 x 16 block of outputs): what a row gets depends on the row and its expert alone, not on
 // the rows it shares a tile with.  The 32-bit mode runs one fused multiply-add chain per output over the inner size
 // ascending.
 #include <math.h>
@@ -227,67 +227,102 @@ struct MoeArgs {
 // branch: the matrix cores ignore the execution mask); rows past them inside a block read the tile's first row and are
 // never stored.
 template <bool GATE_UP, int MB, int DEPTH>
-__global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w,
-                                                       void* __restrict__ out, int ldo) {
-  const int tile = blockIdx.x;
-  if (tile >= a.meta[0]) return;
+__global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* __restrict__ x, int ldx, int x_rows,
+                                                       const bf16_t* __restrict__ w, void* __restrict__ out, int ldo, int max_tiles) {
+  // Workgroups are dealt to the chip's eight dies in turn, and every die has an L2 of its own.  Workgroup L is the
+  // (L / 8)-th of die L % 8; a die takes the blocks of 128 columns c = die, die + 8, ... and, for each, walks the tiles
+  // in order: tiles of one expert follow each other, so a block of an expert's weights is fetched into one L2 once and
+  // serves all of the expert's tiles from there.
+  const int die = blockIdx.x & 7, nth = blockIdx.x >> 3;
+  const int tile = nth % max_tiles, col_block = die + 8 * (nth / max_tiles);
+  if (tile >= a.meta[0] || col_block * 128 >= a.N) return;
   const int wave = wave_index(), lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   const int e = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4]), p0 = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4 + 1]),
             cnt = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4 + 2]);
-  const int n0 = blockIdx.y * 128 + wave * 32;
+  const int n0 = col_block * 128 + wave * 32;
   if (n0 >= a.N) return;                                   // (scalar: the wave's columns lie past the matrix)
   constexpr int NB = GATE_UP ? 4 : 2;
   const int mb_live = (cnt + 15) >> 4;                     // blocks of 16 rows that hold a slot
-  const bf16_t* xr[MB];
+  // Every load goes through a buffer descriptor with a per-lane offset fixed for the whole kernel and the step's offset
+  // in a scalar register: the loop spends no vector instruction on addresses and no branch on a load.  Rows of x are
+  // gathered (a lane's offset names its slot's row); lanes of row blocks without slots and of weight rows past the
+  // matrix point outside their descriptors, read zeros and ask memory for nothing.
+  const int K = a.K;
+  const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((size_t)x_rows * ldx * 2), 0x00020000);
+  int voff_x[MB];
 #pragma unroll
   for (int i = 0; i < MB; ++i) {
     const int q = 16 * i + r;
     const int pq = p0 + (q < cnt ? q : 0);
-    xr[i] = x + (GATE_UP ? (size_t)(a.sorted[pq] / a.top) : (size_t)pq) * ldx + 8 * g;
+    const size_t row = GATE_UP ? (size_t)(a.sorted[pq] / a.top) : (size_t)pq;
+    voff_x[i] = i < mb_live ? (int)((row * ldx + 16 * g) * 2) : 0x7ffffff0;
   }
   // weights of expert e: GATE_UP [2N, K] (gate rows, then up rows), else [N, K]
-  const bf16_t* wr[NB];
+  __amdgpu_buffer_rsrc_t rs_w[NB];
   const size_t wbase = (size_t)e * (GATE_UP ? 2 : 1) * a.N * a.K;
 #pragma unroll
   for (int b = 0; b < NB; ++b) {
     const int half = GATE_UP ? b >> 1 : 0, cb = GATE_UP ? b & 1 : b;
-    const int n = min(n0 + 16 * cb + r, a.N - 1);
-    wr[b] = w + wbase + ((size_t)half * a.N + n) * a.K + 8 * g;
+    const int nb0 = n0 + 16 * cb;
+    const int rows_in = min(16, a.N - nb0);                // (may be <= 0: then nothing of the block is read)
+    rs_w[b] = __builtin_amdgcn_make_buffer_rsrc((void*)(w + wbase + ((size_t)half * a.N + (rows_in > 0 ? nb0 : 0)) * a.K), 0,
+                                                rows_in > 0 ? (int)((size_t)rows_in * a.K * 2) : 0, 0x00020000);
   }
+  const int voff_w = (r * K + 16 * g) * 2;
   f32x4 acc[MB][NB];
 #pragma unroll
   for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int b = 0; b < NB; ++b) acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  const int K = a.K;
-  struct Ops { u32x4 af[MB], bfr[NB]; };
+  const bool tail = (K & 63) != 0;                         // (scalar)
+  // A step covers 64 elements of the inner size: lane (r, g) holds elements k + 16g .. k + 16g + 15 of its row, 32
+  // contiguous bytes, so that a wave's loads take whole 128-byte lines; the first matrix instruction of the step
+  // multiplies every lane's first eight elements, the second its last eight (which elements meet in which instruction
+  // is the same for both operands and for every tile shape, so the sums' bits do not depend on the shape).
+  struct Ops { u32x4 af[MB][2], bfr[NB][2]; };
   auto load = [&](int k, Ops& o) {
-    const bool live = k + 8 * g + 8 <= K;                  // (K is a multiple of 8; past K nothing is asked of memory)
-#pragma unroll
-    for (int i = 0; i < MB; ++i) o.af[i] = (live && i < mb_live) ? *reinterpret_cast<const u32x4*>(xr[i] + k) : zero;
-#pragma unroll
-    for (int b = 0; b < NB; ++b) o.bfr[b] = live ? *reinterpret_cast<const u32x4*>(wr[b] + k) : zero;
-  };
-  auto mma = [&](const Ops& o) {
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
-      if (i < mb_live) {                                   // scalar
+      o.af[i][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff_x[i], k * 2, 0);
+      o.af[i][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff_x[i], k * 2 + 16, 0);
+    }
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-          acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(o.af[i]), as_bf16x8(o.bfr[b]), acc[i][b], 0, 0, 0);
+    for (int b = 0; b < NB; ++b) {
+      o.bfr[b][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_w[b], voff_w, k * 2, 0);
+      o.bfr[b][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_w[b], voff_w, k * 2 + 16, 0);
+    }
+  };
+  auto mma = [&](int k, const Ops& o) {
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+      // (an inner size that is no multiple of 64: what a lane holds past K came from the next row, and counts as zero)
+      const bool live = !tail || k + 16 * g + 8 * hlf + 8 <= K;
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        if (i < mb_live) {                                 // scalar
+          const u32x4 av = live ? o.af[i][hlf] : zero;
+#pragma unroll
+          for (int b = 0; b < NB; ++b)
+            acc[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av), as_bf16x8(live ? o.bfr[b][hlf] : zero), acc[i][b], 0, 0, 0);
+        }
       }
     }
   };
   Ops ring[DEPTH];
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) load(32 * d, ring[d]);
-  for (int k = 0; k < K; k += 32 * DEPTH) {
+  for (int d = 0; d < DEPTH; ++d) load(64 * d, ring[d]);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int k = 0; k < K; k += 64 * DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      if (k + 32 * d < K) {                                // (scalar)
-        mma(ring[d]);
-        load(k + 32 * (d + DEPTH), ring[d]);
+      if (k + 64 * d < K) {                                // (scalar)
+        mma(k + 64 * d, ring[d]);
+        // the refill stays where it is written: left to itself the scheduler moves every load to just before its
+        // use, and the ring holds nothing in flight
+        __builtin_amdgcn_sched_barrier(0);
+        load(k + 64 * (d + DEPTH), ring[d]);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
@@ -345,7 +380,7 @@ __global__ __launch_bounds__(64) void moe_f32_kernel(MoeArgs a, const float* __r
   }
 }
 
-extern "C" int bw_moe_experts(const void* x, int x_is_bf16, int ldx, const void* w, int w_is_bf16, void* out, int ldo,
+extern "C" int bw_moe_experts(const void* x, int x_is_bf16, int ldx, int x_rows, const void* w, int w_is_bf16, void* out, int ldo,
                               const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int slots, int max_tiles, int top,
                               int K, int N, int gate_up, float limit, float alpha, int round_out, void* stream) {
   const int tile_rows = bw_moe_tile_rows(slots);          // (as the plan was made)
@@ -355,13 +390,15 @@ extern "C" int bw_moe_experts(const void* x, int x_is_bf16, int ldx, const void*
   hipStream_t s = (hipStream_t)stream;
   if (x_is_bf16) {
     if (!w_is_bf16 || K % 8 || ldx % 8) return -3;
-    const dim3 grid(max_tiles, (N + 127) / 128);
+    if ((size_t)x_rows * ldx * 2 >= (1ull << 31) || (size_t)16 * K * 2 >= (1ull << 31)) return -2;      // offsets inside a descriptor are 32-bit
+    const int col_blocks = (N + 127) / 128;
+    const dim3 grid((unsigned)(8 * ((col_blocks + 7) / 8) * max_tiles));
     if (tile_rows == 16) {
-      if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, 1, 8>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
-      else hipLaunchKernelGGL((moe_mfma_kernel<false, 1, 12>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+      if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, 1, 4>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
+      else hipLaunchKernelGGL((moe_mfma_kernel<false, 1, 6>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
     } else {
-      if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, MOE_TM / 16, 3>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
-      else hipLaunchKernelGGL((moe_mfma_kernel<false, MOE_TM / 16, 3>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, (const bf16_t*)w, out, ldo);
+      if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, MOE_TM / 16, 2>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
+      else hipLaunchKernelGGL((moe_mfma_kernel<false, MOE_TM / 16, 2>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
     }
     return BW_LAUNCH_CHECK();
   }

@@ -105,7 +105,7 @@ _SIGS = {
     "bw_moe_route": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "bw_moe_max_tiles": [c_int, c_int],
     "bw_moe_plan": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
-    "bw_moe_experts": [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+    "bw_moe_experts": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                        c_int, c_int, c_int, c_float, c_float, c_int, c_void_p],
     "bw_moe_combine": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "bw_shared_key_attention": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int,
@@ -1141,7 +1141,7 @@ def moe_experts(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_slot
     max_tiles = moe_max_tiles(slots, experts)
     if tiles.numel() < 4 * max_tiles or sorted_slots.numel() < slots:
         raise ValueError("moe_experts: the plan's tables are too small")
-    _check(_fn("bw_moe_experts")(x.data_ptr(), xb, x.stride(0), w.data_ptr(), wb, out.data_ptr(), out.stride(0), sorted_slots.data_ptr(),
+    _check(_fn("bw_moe_experts")(x.data_ptr(), xb, x.stride(0), x.shape[0], w.data_ptr(), wb, out.data_ptr(), out.stride(0), sorted_slots.data_ptr(),
                                  tiles.data_ptr(), meta.data_ptr(), slots, max_tiles, top, K, N, int(gate_up), float(limit), float(alpha),
                                  int(round_out), _stream()), "moe_experts")
 
