@@ -114,7 +114,7 @@ def sepedra_shape(width: int, expert_ff: int, groups: int, experts: int = 32, to
         att = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5, "rot": rot}
         layers.append({"type": "attention", "mixer": dict(att), "mlp": mlp})
         layers.append({"type": "attention", "mixer": dict(att, kv_from=4 * g + 2), "mlp": mlp})
-    return {"architecture": "Sepedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+    return {"architecture": "Sepedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 50.0,
             "layers": layers, "max_positions": 16384, "eos_token_id": 2}
 
 

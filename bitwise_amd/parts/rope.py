@@ -62,7 +62,7 @@ class PairRotaryTable(PositionEncoding):
     l = 2 pi / f, a frequency stays where l < original / high, becomes f / factor where l > original / low, and in
     between is (1 - s) f / factor + s f with s = (original / l - low) / (high - low).
     Frequencies and angles are computed in double precision on the host and the cosines and sines rounded once to
-    32-bit.  No checkpoint tensors.  The tables are those of the base contract, [positions, dims / 2]; which
+    32-bit.  No checkpoint tensors.  The tables are what the base class promises, [positions, dims / 2]; which
     elements a column pairs is the mixer's business (``layout``)."""
 
     graph_safe = True
