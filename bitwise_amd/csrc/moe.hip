@@ -395,8 +395,11 @@ __global__ __launch_bounds__(256) void moe_lds_kernel(MoeArgs a, const bf16_t* _
     }
   }
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  u32x4 regs[NCH];
-  auto fetch = [&](int k) {
+  // two sets of registers: the loads of the next step and of the one after it are in flight while a step is multiplied
+  // (every weight comes from memory once, so what hides the memory's latency is the bytes a compute unit has asked for)
+  u32x4 regs_a[NCH], regs_b[NCH];
+  auto fetch = [&](int k, u32x4 (&regs)[NCH]) {
+    if (k >= K) return;                                    // (scalar)
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       // (a thread's chunk j lies in rows 32 j .. 32 j + 31: x rows for the first TM / 32 chunks, weight rows after)
@@ -404,7 +407,8 @@ __global__ __launch_bounds__(256) void moe_lds_kernel(MoeArgs a, const bf16_t* _
                             : __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff[j], k * 2, 0);
     }
   };
-  auto stash = [&](int k, int stage) {
+  auto stash = [&](int k, int stage, const u32x4 (&regs)[NCH]) {
+    if (k >= K) return;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       const int part = (tid + 256 * j) & 7;
@@ -425,13 +429,7 @@ __global__ __launch_bounds__(256) void moe_lds_kernel(MoeArgs a, const bf16_t* _
     const int half = GATE_UP ? b >> 2 : 0, cb = b & 3;
     b_off[b] = (TM + 128 * half + 64 * wc + 16 * cb + r) * MOE_LDS_STRIDE + 32 * g;
   }
-  fetch(0);
-  stash(0, 0);
-  __syncthreads();
-  int stage = 0;
-  for (int k = 0; k < K; k += 64) {
-    const bool more = k + 64 < K;                          // (scalar)
-    if (more) fetch(k + 64);
+  auto multiply = [&](int stage) {
     const unsigned char* base = moe_lds + stage * STAGE;
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
@@ -448,9 +446,25 @@ __global__ __launch_bounds__(256) void moe_lds_kernel(MoeArgs a, const bf16_t* _
         }
       }
     }
-    if (more) stash(k + 64, stage ^ 1);
+  };
+  fetch(0, regs_a);
+  fetch(64, regs_b);
+  stash(0, 0, regs_a);
+  fetch(128, regs_a);
+  __syncthreads();
+  // step k is multiplied from stage 0 while regs_b (step k + 64) goes to stage 1 and is asked for again three steps ahead;
+  // then the same with the roles swapped
+  for (int k = 0; k < K; k += 128) {
+    multiply(0);
+    stash(k + 64, 1, regs_b);
+    fetch(k + 192, regs_b);
     __syncthreads();
-    stage ^= 1;
+    if (k + 64 < K) {                                      // (scalar)
+      multiply(1);
+      stash(k + 128, 0, regs_a);
+      fetch(k + 256, regs_a);
+      __syncthreads();
+    }
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
