@@ -127,7 +127,7 @@ int bw_shared_key_attention_mfma(const void* q, int ldq, const int32_t* position
 // Mixers that convolve their projections over a few tokens, gate their outputs or carry a gated recurrence per channel,
 // and row operations of layers whose norm sits behind the sublayer (gated_mix.hip).  sink (the attention entry points
 // above): a score per head that joins the softmax's denominator and has no value, or null.
-int bw_causal_conv(const float* x, int ldx, const void* w, const void* bias, int w_is_bf16, int taps, int channels,
+int bw_causal_conv(const float* x, int ldx, const float* in_bias, const void* w, const void* bias, int w_is_bf16, int taps, int channels,
                    float* state, long long state_ld, const int32_t* seq_rows, const int32_t* slots,
                    const int32_t* positions, int nseq, int max_seq_rows, float* out, int ldo, void* stream);
 int bw_pair_rope_unit(const float* src, int lds, const int32_t* positions, const int32_t* row_seq,
@@ -138,16 +138,20 @@ int bw_pair_rope_unit(const float* src, int lds, const int32_t* positions, const
 int bw_gate_mul(const void* av, int a_is_bf16, int lda, int hd, const float* g, int ldg, void* out, int out_is_bf16,
                 int ldo, int rows, int heads, int vdim, void* stream);
 // (y and gates are overwritten: y by its activation, the gates' logits by the recurrence's factor and addend)
-int bw_rglru_scan(float* y, int ldy, const float* u, int ldu, float* gates, int ldg, const float* ra_bias,
+int bw_rglru_scan(float* y, int ldy, const float* y_bias, const float* u, int ldu, float* gates, int ldg, const float* ra_bias,
                   const float* ri_bias, const float* decay, float* state, long long state_ld, void* out,
                   int out_is_bf16, int ldo, const int32_t* seq_rows, const int32_t* slots, const int32_t* positions,
                   int nseq, int rows, int channels, int bs, void* stream);
+// place, wts, top (optional): row r of the normed operand is sum_j wts[r][j] * y[place[r][j]] instead of y[r]
 int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, void* rounded, int ldr,
-                int rows, int dim, float eps, void* stream);
+                int rows, int dim, float eps, const int32_t* place, const float* wts, int top, void* stream);
 int bw_softcap(float* x, int ld, int rows, int cols, float cap, void* stream);
 // A feed-forward of routed experts (moe.hip).
 int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
                  float* wts, void* stream);
+// route, then plan; one launch for steps of up to 16 rows
+int bw_moe_route_plan(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
+                      float* wts, int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream);
 int bw_moe_max_tiles(int slots, int experts);
 int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* sorted, int32_t* place, int32_t* tiles,
                 int32_t* meta, void* stream);

@@ -35,7 +35,8 @@ __device__ __forceinline__ float gm_sigmoid(float x) { return 1.0f / (1.0f + bw_
 struct ConvArgs {
   const float* x;        // [rows, ldx]: channel c at column c
   const void* w;         // [channels, taps]
-  const void* bias;      // [channels] or null
+  const void* bias;      // [channels] or null: added to every output
+  const float* in_bias;  // [channels] or null: added to every input on its way in (the state keeps inputs with it)
   float* state;          // [slots, state_ld]: [taps - 1][channels] at the pointer, oldest first
   float* out;            // [rows, ldo]
   const int32_t* seq_rows;
@@ -59,6 +60,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
   const float bias = a.bias != nullptr ? gm_load(reinterpret_cast<const WT*>(a.bias) + c) : 0.0f;
   float* st = a.state + (size_t)slot * a.state_ld + c;
   const float* x = a.x + (size_t)first * a.ldx + c;
+  const float ib = a.in_bias != nullptr ? a.in_bias[c] : 0.0f;
   // only the request's first chunk reaches back before the portion, and only its threads touch the slot
   float old[P];
 #pragma unroll
@@ -67,11 +69,11 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
 #pragma unroll
   for (int j = 0; j < P; ++j) {
     const int idx = t0 - (TAPS - 1) + j;
-    win[j] = idx >= 0 ? x[(size_t)idx * a.ldx] : old[(TAPS - 1 + idx) < 0 ? 0 : (TAPS - 1 + idx)];
+    win[j] = idx >= 0 ? x[(size_t)idx * a.ldx] + ib : old[(TAPS - 1 + idx) < 0 ? 0 : (TAPS - 1 + idx)];
   }
   float* o = a.out + (size_t)first * a.ldo + c;
   for (int t = t0; t < t1; ++t) {
-    const float cur = x[(size_t)t * a.ldx];
+    const float cur = x[(size_t)t * a.ldx] + ib;
     float acc = 0.0f;
     if constexpr (TAPS > 1) {
 #pragma unroll
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
     for (int j = 0; j < TAPS - 1; ++j) {
       const int idx = n - (TAPS - 1) + j;
       float v = 0.0f;
-      if (idx >= 0) v = x[(size_t)idx * a.ldx];
+      if (idx >= 0) v = x[(size_t)idx * a.ldx] + ib;
       else {
 #pragma unroll
         for (int q = 0; q < P; ++q) v = (q == TAPS - 1 + idx) ? old[q] : v;
@@ -112,12 +114,12 @@ static int conv_launch(const ConvArgs& a, int taps, dim3 grid, hipStream_t s) {
   return BW_LAUNCH_CHECK();
 }
 
-extern "C" int bw_causal_conv(const float* x, int ldx, const void* w, const void* bias, int w_is_bf16, int taps, int channels,
+extern "C" int bw_causal_conv(const float* x, int ldx, const float* in_bias, const void* w, const void* bias, int w_is_bf16, int taps, int channels,
                               float* state, long long state_ld, const int32_t* seq_rows, const int32_t* slots,
                               const int32_t* positions, int nseq, int max_seq_rows, float* out, int ldo, void* stream) {
   if (nseq <= 0 || channels <= 0 || max_seq_rows <= 0) return 0;
   if (taps < 1 || taps > CONV_MAX_TAPS || (taps > 1 && state == nullptr)) return -2;
-  ConvArgs a{x, w, bias, state, out, seq_rows, slots, positions, state_ld, ldx, ldo, channels};
+  ConvArgs a{x, w, bias, in_bias, state, out, seq_rows, slots, positions, state_ld, ldx, ldo, channels};
   const dim3 grid((channels + 255) / 256, nseq, (max_seq_rows + CONV_CHUNK - 1) / CONV_CHUNK);
   if (grid.y > 65535 || grid.z > 65535) return -2;
   return w_is_bf16 ? conv_launch<bf16_t>(a, taps, grid, (hipStream_t)stream) : conv_launch<float>(a, taps, grid, (hipStream_t)stream);
@@ -260,6 +262,7 @@ struct RglruArgs {
   const float* ra_bias;   // [channels]
   const float* ri_bias;
   const float* decay;     // [channels]: c = -scale * softplus(lambda), so that log a = c * r
+  const float* y_bias;    // [channels] or null: added to the gate branch before its activation
   float* state;           // [slots, state_ld]: S [channels] at the pointer
   void* out;              // [rows, ldo]
   const int32_t* seq_rows;
@@ -295,7 +298,7 @@ __global__ __launch_bounds__(256) void rglru_terms_kernel(RglruArgs p, int rows)
   rglru_terms(zr[0], zr[p.bs], p.u[(size_t)row * p.ldu + c], p.ra_bias[c], p.ri_bias[c], p.decay[c], a, b);
   zr[0] = a;
   zr[p.bs] = b;
-  *yy = gm_gelu_tanh(*yy);
+  *yy = gm_gelu_tanh(p.y_bias != nullptr ? *yy + p.y_bias[c] : *yy);
 }
 
 template <typename TO>
@@ -333,13 +336,13 @@ __global__ __launch_bounds__(64) void rglru_scan_kernel(RglruArgs p) {
   *st = S;
 }
 
-extern "C" int bw_rglru_scan(float* y, int ldy, const float* u, int ldu, float* gates, int ldg, const float* ra_bias,
+extern "C" int bw_rglru_scan(float* y, int ldy, const float* y_bias, const float* u, int ldu, float* gates, int ldg, const float* ra_bias,
                              const float* ri_bias, const float* decay, float* state, long long state_ld, void* out,
                              int out_is_bf16, int ldo, const int32_t* seq_rows, const int32_t* slots, const int32_t* positions,
                              int nseq, int rows, int channels, int bs, void* stream) {
   if (nseq <= 0 || channels <= 0 || rows <= 0) return 0;
   if (bs <= 0 || channels % bs || nseq > 65535 || rows > 65535) return -2;
-  RglruArgs p{y, u, gates, ra_bias, ri_bias, decay, state, out, seq_rows, slots, positions, state_ld, ldy, ldu, ldg, ldo, channels, bs};
+  RglruArgs p{y, u, gates, ra_bias, ri_bias, decay, y_bias, state, out, seq_rows, slots, positions, state_ld, ldy, ldu, ldg, ldo, channels, bs};
   hipLaunchKernelGGL(rglru_terms_kernel, dim3((channels + 255) / 256, rows), dim3(256), 0, (hipStream_t)stream, p, rows);
   const dim3 grid((channels + 63) / 64, nseq);
   if (out_is_bf16) hipLaunchKernelGGL(rglru_scan_kernel<bf16_t>, grid, dim3(64), 0, (hipStream_t)stream, p);
@@ -352,12 +355,22 @@ extern "C" int bw_rglru_scan(float* y, int ldy, const float* u, int ldu, float* 
 // A workgroup a row.  Thread t owns elements t, t + 256, ...; its sum of squares is one chain over them, the waves'
 // sums are joined by the butterflies of wave_sum and the four of them added in wave order: the same order for every
 // row of every launch.  rounded (optional): the new row once more, rounded to bfloat16, for the next sublayer's products.
+// place, wts (optional): y is then not the row itself but a table of rows of which this row is a weighted sum,
+// y_row[e] = sum_j wts[row][j] * y[place[row][j]][e], j ascending, one chain an element (what a feed-forward of routed
+// experts leaves: its choices' outputs by sorted place); the sum is formed here instead of by a launch of its own.
 template <typename WT>
 __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__ y, int ldy, const WT* __restrict__ w, float* __restrict__ x,
-                                                       int ldx, bf16_t* __restrict__ rounded, int ldr, int dim, float eps) {
+                                                       int ldx, bf16_t* __restrict__ rounded, int ldr, int dim, float eps,
+                                                       const int32_t* __restrict__ place, const float* __restrict__ wts, int top) {
   __shared__ float part[4];
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* yr = y + (size_t)row * ldy;
+  auto value = [&](int e) -> float {
+    if (place == nullptr) return yr[e];
+    float acc = 0.0f;
+    for (int j = 0; j < top; ++j) acc = fmaf(wts[(size_t)row * top + j], y[(size_t)place[(size_t)row * top + j] * ldy + e], acc);
+    return acc;
+  };
   constexpr int MAXV = 8;                       // rows of up to 256 * MAXV elements keep their values in registers
   float v[MAXV];
   float acc = 0.0f;
@@ -365,12 +378,15 @@ __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) {
       const int e = tid + 256 * j;
-      v[j] = e < dim ? yr[e] : 0.0f;
+      v[j] = e < dim ? value(e) : 0.0f;
     }
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) acc = fmaf(v[j], v[j], acc);
   } else {
-    for (int e = tid; e < dim; e += 256) acc = fmaf(yr[e], yr[e], acc);
+    for (int e = tid; e < dim; e += 256) {
+      const float ye = value(e);
+      acc = fmaf(ye, ye, acc);
+    }
   }
   acc = wave_sum(acc);
   if ((tid & 63) == 0) part[tid >> 6] = acc;
@@ -390,7 +406,7 @@ __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__
     }
   } else {
     for (int e = tid; e < dim; e += 256) {
-      const float nx = xr[e] + (yr[e] * inv) * gm_load(w + e);
+      const float nx = xr[e] + (value(e) * inv) * gm_load(w + e);
       xr[e] = nx;
       if (rounded != nullptr) rounded[(size_t)row * ldr + e] = f32_to_bf16(nx);
     }
@@ -398,13 +414,13 @@ __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__
 }
 
 extern "C" int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, void* rounded, int ldr,
-                           int rows, int dim, float eps, void* stream) {
+                           int rows, int dim, float eps, const int32_t* place, const float* wts, int top, void* stream) {
   if (rows <= 0) return 0;
   const dim3 grid(rows);
   if (w_is_bf16)
-    hipLaunchKernelGGL(norm_add_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const bf16_t*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps);
+    hipLaunchKernelGGL(norm_add_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const bf16_t*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps, place, wts, top);
   else
-    hipLaunchKernelGGL(norm_add_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const float*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps);
+    hipLaunchKernelGGL(norm_add_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const float*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps, place, wts, top);
   return BW_LAUNCH_CHECK();
 }
 

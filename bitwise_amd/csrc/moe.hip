@@ -5,7 +5,7 @@
 //             the `top` best of those are the row's experts, weighted by their scores as they are.  Ties go to the
 //             lower index.  All 32-bit.
 //   plan:     the step's (row, choice) pairs ("slots") sorted by expert into runs, and the runs cut into tiles of
-//             MOE_TM slots: every tile belongs to one expert.  Built on the device; the products' grids are sized for
+//             16 or 128 slots (steps of few or of many slots): every tile belongs to one expert.  Built on the device; the products' grids are sized for
 //             the worst case and tiles past the last return at once.
 //   gate_up:  per tile, G = X W_gate^T and U = X W_up^T of its expert, then h = min(G, limit) * sigmoid(alpha * min(G, limit))
 //             * (clamp(U, -limit, limit) + 1), stored by the slot's place in the sorted order
@@ -39,14 +39,9 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
   }
 }
 
-// A wave a row.  LDS per wave: scores [E], group scores [count], allowed [count].
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, int rows, int E, int top, int count,
-                                                        int keep, int32_t* __restrict__ ids, float* __restrict__ wts) {
-  extern __shared__ float route_lds[];
-  const int wave = wave_index(), lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + wave;
-  if (row >= rows) return;
-  float* s = route_lds + (size_t)wave * (E + 2 * count);
+// A wave a row.  LDS of the wave: scores [E], group scores [count], allowed [count].
+__device__ __forceinline__ void route_row(const float* __restrict__ logits, int ld, int row, int E, int top, int count, int keep,
+                                          int32_t* __restrict__ ids, float* __restrict__ wts, float* s, int lane) {
   float* gs = s + E;
   float* allowed = gs + count;
   const float* z = logits + (size_t)row * ld;
@@ -98,6 +93,15 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   }
 }
 
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, int rows, int E, int top, int count,
+                                                        int keep, int32_t* __restrict__ ids, float* __restrict__ wts) {
+  extern __shared__ float route_lds[];
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  route_row(logits, ld, row, E, top, count, keep, ids, wts, route_lds + (size_t)wave * (E + 2 * count), lane);
+}
+
 extern "C" int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
                             float* wts, void* stream) {
   if (rows <= 0) return 0;
@@ -117,10 +121,9 @@ extern "C" int bw_moe_route(const float* logits, int ld, int rows, int experts, 
 // slots (from LDS, where the workgroup has put them if they fit) and counts those of expert e; after a prefix over
 // segments and experts it walks the segment again and hands out places.  Within an expert's run the slots ascend, so
 // the plan is the same from run to run.
-__global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ ids, int n, int E, int segs, int tm, int staged,
-                                                        int32_t* __restrict__ sorted, int32_t* __restrict__ place,
-                                                        int32_t* __restrict__ tiles, int32_t* __restrict__ meta) {
-  extern __shared__ int plan_ids[];     // [n] if staged
+__device__ __forceinline__ void plan_body(const int32_t* __restrict__ ids, int n, int E, int segs, int tm, int staged, int* plan_ids,
+                                          int32_t* __restrict__ sorted, int32_t* __restrict__ place, int32_t* __restrict__ tiles,
+                                          int32_t* __restrict__ meta) {
   __shared__ int seg_count[1024];       // [expert][segment]; after the prefix: slots of the expert in earlier segments
   __shared__ int counts[MOE_MAX_EXPERTS], start[MOE_MAX_EXPERTS], tile0[MOE_MAX_EXPERTS];
   const int tid = threadIdx.x;
@@ -181,6 +184,25 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restric
   }
 }
 
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ ids, int n, int E, int segs, int tm, int staged,
+                                                        int32_t* __restrict__ sorted, int32_t* __restrict__ place,
+                                                        int32_t* __restrict__ tiles, int32_t* __restrict__ meta) {
+  extern __shared__ int plan_lds[];     // [n] if staged
+  plan_body(ids, n, E, segs, tm, staged, plan_lds, sorted, place, tiles, meta);
+}
+
+// Steps of up to 16 rows: route (a wave a row) and plan in one launch of one workgroup.
+__global__ __launch_bounds__(1024) void moe_route_plan_kernel(const float* __restrict__ logits, int ld, int rows, int E, int top, int count,
+                                                              int keep, int32_t* __restrict__ ids, float* __restrict__ wts, int segs,
+                                                              int tm, int32_t* __restrict__ sorted, int32_t* __restrict__ place,
+                                                              int32_t* __restrict__ tiles, int32_t* __restrict__ meta) {
+  extern __shared__ float both_lds[];   // the waves' routing tables, then the plan's slots
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  if (wave < rows) route_row(logits, ld, wave, E, top, count, keep, ids, wts, both_lds + (size_t)wave * (E + 2 * count), lane);
+  __syncthreads();                      // (the rows' choices, written to memory by their waves, are visible to the workgroup)
+  plan_body(ids, rows * top, E, segs, tm, 1, reinterpret_cast<int*>(both_lds + (size_t)rows * (E + 2 * count)), sorted, place, tiles, meta);
+}
+
 // Slots a tile: few slots a step (decoded tokens) get tiles of 16, whose kernel keeps many steps of weights in flight;
 // prompt portions get tiles of 128, which a workgroup stages in LDS.
 extern "C" int bw_moe_tile_rows(int slots) { return slots <= MOE_SMALL_SLOTS ? 16 : MOE_TM; }
@@ -198,6 +220,22 @@ extern "C" int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* 
   const int staged = slots <= 12 * 1024;
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), staged ? (size_t)slots * sizeof(int) : 0, (hipStream_t)stream, ids, slots,
                      experts, segs, bw_moe_tile_rows(slots), staged, sorted, place, tiles, meta);
+  return BW_LAUNCH_CHECK();
+}
+
+extern "C" int bw_moe_route_plan(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
+                                 float* wts, int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream) {
+  if (rows <= 0) return 0;
+  const size_t bytes = ((size_t)rows * (experts + 2 * groups) + (size_t)rows * top) * sizeof(float);
+  if (rows > 16 || bytes > 48 * 1024) {
+    const int rc = bw_moe_route(logits, ld, rows, experts, top, groups, keep, ids, wts, stream);
+    return rc != 0 ? rc : bw_moe_plan(ids, rows * top, experts, sorted, place, tiles, meta, stream);
+  }
+  if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || groups < 1 || experts % groups || keep < 1 || keep > groups ||
+      top > keep * (experts / groups))
+    return -2;
+  hipLaunchKernelGGL(moe_route_plan_kernel, dim3(1), dim3(1024), bytes, (hipStream_t)stream, logits, ld, rows, experts, top, groups, keep,
+                     ids, wts, 1024 / experts, bw_moe_tile_rows(rows * top), sorted, place, tiles, meta);
   return BW_LAUNCH_CHECK();
 }
 
@@ -219,14 +257,14 @@ struct MoeArgs {
   float limit, alpha;
 };
 
-// A workgroup of four waves per (tile of MOE_TM slots, 128 output columns); a wave owns 32 columns, for GATE_UP of
+// A workgroup of four waves per (tile of 16 MB slots, 128 output columns); a wave owns 32 columns, for GATE_UP of
 // the gate and of the up matrix both, and all of the tile's rows.  Operands go from memory straight into registers: lane
 // (r, g) holds row r's (or column r's) elements k + 8g .. k + 8g + 7; a ring of DEPTH sets of operand registers keeps as
 // many steps of the inner size in flight.  MB blocks of 16 rows a tile: 1 with a deep ring for the few rows of decoded
 // tokens, where the weights stream from memory once and nothing is reused (prompt portions: moe_lds_kernel below).  Blocks of 16 rows past the tile's slots are skipped (a scalar
 // branch: the matrix cores ignore the execution mask); rows past them inside a block read the tile's first row and are
 // never stored.
-template <bool GATE_UP, int MB, int DEPTH>
+template <bool GATE_UP, int MB, int DEPTH, int CW>
 __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* __restrict__ x, int ldx, int x_rows,
                                                        const bf16_t* __restrict__ w, void* __restrict__ out, int ldo, int max_tiles) {
   // Workgroups are dealt to the chip's eight dies in turn, and every die has an L2 of its own.  Workgroup L is the
@@ -235,13 +273,13 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* 
   // serves all of the expert's tiles from there.
   const int die = blockIdx.x & 7, nth = blockIdx.x >> 3;
   const int tile = nth % max_tiles, col_block = die + 8 * (nth / max_tiles);
-  if (tile >= a.meta[0] || col_block * 128 >= a.N) return;
+  if (tile >= a.meta[0] || col_block * (4 * CW) >= a.N) return;
   const int wave = wave_index(), lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   const int e = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4]), p0 = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4 + 1]),
             cnt = __builtin_amdgcn_readfirstlane(a.tiles[tile * 4 + 2]);
-  const int n0 = col_block * 128 + wave * 32;
-  if (n0 >= a.N) return;                                   // (scalar: the wave's columns lie past the matrix)
-  constexpr int NB = GATE_UP ? 4 : 2;
+  const int n0 = col_block * (4 * CW) + wave * CW;         // CW columns a wave (32, or 16 where a step has very few slots
+  if (n0 >= a.N) return;                                   // and more workgroups are worth more than wider ones)
+  constexpr int CB = CW / 16, NB = GATE_UP ? 2 * CB : CB;
   const int mb_live = (cnt + 15) >> 4;                     // blocks of 16 rows that hold a slot
   // Every load goes through a buffer descriptor with a per-lane offset fixed for the whole kernel and the step's offset
   // in a scalar register: the loop spends no vector instruction on addresses and no branch on a load.  Rows of x are
@@ -262,7 +300,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* 
   const size_t wbase = (size_t)e * (GATE_UP ? 2 : 1) * a.N * a.K;
 #pragma unroll
   for (int b = 0; b < NB; ++b) {
-    const int half = GATE_UP ? b >> 1 : 0, cb = GATE_UP ? b & 1 : b;
+    const int half = GATE_UP ? b / CB : 0, cb = GATE_UP ? b % CB : b;
     const int nb0 = n0 + 16 * cb;
     const int rows_in = min(16, a.N - nb0);                // (may be <= 0: then nothing of the block is read)
     rs_w[b] = __builtin_amdgcn_make_buffer_rsrc((void*)(w + wbase + ((size_t)half * a.N + (rows_in > 0 ? nb0 : 0)) * a.K), 0,
@@ -334,11 +372,11 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(MoeArgs a, const bf16_t* 
       const int m = 16 * i + 4 * g + q;
       if (m >= cnt) continue;
 #pragma unroll
-      for (int cb = 0; cb < 2; ++cb) {
+      for (int cb = 0; cb < CB; ++cb) {
         const int n = n0 + 16 * cb + r;
         if (n >= a.N) continue;
         if constexpr (GATE_UP)
-          reinterpret_cast<bf16_t*>(out)[(size_t)(p0 + m) * ldo + n] = f32_to_bf16(moe_act(acc[i][cb][q], acc[i][2 + cb][q], a.limit, a.alpha));
+          reinterpret_cast<bf16_t*>(out)[(size_t)(p0 + m) * ldo + n] = f32_to_bf16(moe_act(acc[i][cb][q], acc[i][CB + cb][q], a.limit, a.alpha));
         else
           reinterpret_cast<float*>(out)[(size_t)(p0 + m) * ldo + n] = acc[i][cb][q];
       }
@@ -545,11 +583,18 @@ extern "C" int bw_moe_experts(const void* x, int x_is_bf16, int ldx, int x_rows,
   if (x_is_bf16) {
     if (!w_is_bf16 || K % 8 || ldx % 8) return -3;
     if ((size_t)x_rows * ldx * 2 >= (1ull << 31) || (size_t)16 * K * 2 >= (1ull << 31)) return -2;      // offsets inside a descriptor are 32-bit
-    const int col_blocks = (N + 127) / 128;
-    const dim3 grid((unsigned)(8 * ((col_blocks + 7) / 8) * max_tiles));
     if (tile_rows == 16) {
-      if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, 1, 4>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
-      else hipLaunchKernelGGL((moe_mfma_kernel<false, 1, 6>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
+      // very few slots (a step of up to 16 rows of four experts): 16 columns a wave, twice the workgroups
+      const int cw = slots <= 64 ? 16 : 32;
+      const int col_blocks = (N + 4 * cw - 1) / (4 * cw);
+      const dim3 grid((unsigned)(8 * ((col_blocks + 7) / 8) * max_tiles));
+      if (cw == 16) {
+        if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, 1, 6, 16>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
+        else hipLaunchKernelGGL((moe_mfma_kernel<false, 1, 8, 16>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
+      } else {
+        if (gate_up) hipLaunchKernelGGL((moe_mfma_kernel<true, 1, 4, 32>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
+        else hipLaunchKernelGGL((moe_mfma_kernel<false, 1, 6, 32>), grid, dim3(256), 0, s, a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles);
+      }
     } else {
       if ((size_t)2 * N * K * 2 >= (1ull << 31)) return -2;
       return gate_up ? moe_lds_launch<true>(a, (const bf16_t*)x, ldx, x_rows, (const bf16_t*)w, out, ldo, max_tiles, s)

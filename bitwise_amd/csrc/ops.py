@@ -92,17 +92,20 @@ _SIGS = {
                        c_void_p],
     "bw_headwise_linear": [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
                            c_int, c_void_p],
-    "bw_causal_conv": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_longlong, c_void_p, c_void_p,
+    "bw_causal_conv": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_longlong, c_void_p, c_void_p,
                        c_void_p, c_int, c_int, c_void_p, c_int, c_void_p],
     "bw_pair_rope_unit": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                           c_int, c_void_p],
     "bw_gate_mul": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "bw_rglru_scan": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
+    "bw_rglru_scan": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
                       c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-    "bw_norm_add": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+    "bw_norm_add": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
+                    c_int, c_void_p],
     "bw_softcap": [c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "bw_moe_route": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "bw_moe_route_plan": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_void_p],
     "bw_moe_max_tiles": [c_int, c_int],
     "bw_moe_plan": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_moe_experts": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -947,11 +950,12 @@ CONV_MAX_TAPS = 8
 
 def causal_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
                 seq_rows: torch.Tensor, slots: torch.Tensor, positions: torch.Tensor, nseq: int, max_seq_rows: int,
-                out: torch.Tensor) -> None:
+                out: torch.Tensor, in_bias: Optional[torch.Tensor] = None) -> None:
     """out[t, c] = sum_j weight[c, j] * x[t - taps + 1 + j, c] (+ bias[c]) along every request's rows, the inputs before a
     portion's first row taken from ``state`` [slots, >= (taps - 1) * channels] (a view may start inside a wider slot),
     which then receives the portion's last taps - 1 inputs.  ``x`` [rows, >= channels] float32 (rows apart by its
-    stride), ``out`` likewise.  ``max_seq_rows``: the most rows a request brings in this step."""
+    stride), ``out`` likewise.  ``max_seq_rows``: the most rows a request brings in this step.  ``in_bias`` [channels]
+    float32: added to every input on its way in (a projection's bias; the state then keeps inputs with it)."""
     if x.dtype != torch.float32 or out.dtype != torch.float32 or x.stride(1) != 1 or out.stride(1) != 1 or not (x.is_cuda and out.is_cuda):
         raise ValueError("causal_conv: x and out must be float32 GPU matrices with contiguous rows")
     if weight.dim() != 2 or not weight.is_cuda or not weight.is_contiguous():
@@ -973,7 +977,11 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
         if state is None or state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < (taps - 1) * channels:
             raise ValueError(f"causal_conv: a state slot needs {(taps - 1) * channels} float32 elements")
         sp, sld = state.data_ptr(), state.stride(0)
-    _check(_fn("bw_causal_conv")(x.data_ptr(), x.stride(0), weight.data_ptr(), 0 if bias is None else bias.data_ptr(), wb, taps,
+    if in_bias is not None:
+        _need(in_bias, torch.float32, "in_bias")
+        if in_bias.numel() != channels:
+            raise ValueError("causal_conv: in_bias must be [channels]")
+    _check(_fn("bw_causal_conv")(x.data_ptr(), x.stride(0), 0 if in_bias is None else in_bias.data_ptr(), weight.data_ptr(), 0 if bias is None else bias.data_ptr(), wb, taps,
                                  channels, sp, sld, seq_rows.data_ptr(), slots.data_ptr(), positions.data_ptr(), int(nseq),
                                  int(max_seq_rows), out.data_ptr(), out.stride(0), _stream()), "causal_conv")
 
@@ -1031,7 +1039,8 @@ def gate_mul(av: torch.Tensor, head_size: int, g: torch.Tensor, out: torch.Tenso
 
 def rglru_scan(y: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, ra_bias: torch.Tensor, ri_bias: torch.Tensor,
                decay: torch.Tensor, state: torch.Tensor, out: torch.Tensor, seq_rows: torch.Tensor, slots: torch.Tensor,
-               positions: torch.Tensor, nseq: int, rows: int, channels: int, block: int) -> None:
+               positions: torch.Tensor, nseq: int, rows: int, channels: int, block: int,
+               y_bias: Optional[torch.Tensor] = None) -> None:
     """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) * i_t * u_t per channel along every request's rows, from and to ``state``
     [slots, >= channels]; a_t = exp(decay * r_t), r_t = sigmoid(gate logits + ra_bias), i_t likewise with ri_bias;
     ``gates`` [rows, channels/block * 2*block]: per block its recurrence-gate logits, then its input-gate logits;
@@ -1051,28 +1060,42 @@ def rglru_scan(y: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, ra_bias: t
         raise ValueError("rglru_scan: widths do not fit the channels")
     if seq_rows.numel() < 2 * nseq or slots.numel() < nseq or positions.numel() < rows or min(y.shape[0], u.shape[0], gates.shape[0], out.shape[0]) < rows:
         raise ValueError("rglru_scan: fewer request records than requests, or buffers shorter than the rows")
-    _check(_fn("bw_rglru_scan")(y.data_ptr(), y.stride(0), u.data_ptr(), u.stride(0), gates.data_ptr(), gates.stride(0),
+    if y_bias is not None:
+        _need(y_bias, torch.float32, "y_bias")
+        if y_bias.numel() != channels:
+            raise ValueError("rglru_scan: y_bias needs an element per channel")
+    _check(_fn("bw_rglru_scan")(y.data_ptr(), y.stride(0), 0 if y_bias is None else y_bias.data_ptr(), u.data_ptr(), u.stride(0), gates.data_ptr(), gates.stride(0),
                                 ra_bias.data_ptr(), ri_bias.data_ptr(), decay.data_ptr(), state.data_ptr(), state.stride(0),
                                 out.data_ptr(), _act_out(out, "out"), out.stride(0), seq_rows.data_ptr(), slots.data_ptr(),
                                 positions.data_ptr(), int(nseq), int(rows), channels, block, _stream()), "rglru_scan")
 
 
 def norm_add(y: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, rows: int, eps: float,
-             rounded: Optional[torch.Tensor] = None) -> None:
+             rounded: Optional[torch.Tensor] = None, combine: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None) -> None:
     """x[:rows] += y / sqrt(mean(y^2) + eps) * weight, all 32-bit.  ``rounded`` (bfloat16, x's shape): also receives the new
-    rows rounded, for products that follow."""
+    rows rounded, for products that follow.  ``combine`` = (place, wts, top): row r of the normed operand is
+    sum_j wts[r, j] * y[place[r*top + j]] (j ascending, the chain of ``moe_combine``) instead of y[r]."""
     _need(y, torch.float32, "y")
     _need(x, torch.float32, "x")
     dim = x.shape[1]
-    if y.shape[1] != dim or weight.numel() != dim or not weight.is_cuda or min(x.shape[0], y.shape[0]) < rows:
+    if y.shape[1] != dim or weight.numel() != dim or not weight.is_cuda or x.shape[0] < rows or (combine is None and y.shape[0] < rows):
         raise ValueError("norm_add: y, weight and x do not fit")
+    place = wts = None
+    top = 0
+    if combine is not None:
+        place, wts, top = combine
+        _need(place, torch.int32, "place")
+        _need(wts, torch.float32, "wts")
+        if place.numel() < rows * top or wts.numel() < rows * top or top < 1:
+            raise ValueError("norm_add: the combination's tables are shorter than the rows")
     if rounded is not None:
         _need(rounded, torch.bfloat16, "rounded")
         if rounded.shape[1] != dim or rounded.shape[0] < rows:
             raise ValueError("norm_add: the rounded copy does not fit")
     _check(_fn("bw_norm_add")(y.data_ptr(), y.stride(0), weight.data_ptr(), _is_bf16(weight, "weight"), x.data_ptr(), x.stride(0),
                               0 if rounded is None else rounded.data_ptr(), 0 if rounded is None else rounded.stride(0),
-                              rows, dim, float(eps), _stream()), "norm_add")
+                              rows, dim, float(eps), 0 if place is None else place.data_ptr(), 0 if wts is None else wts.data_ptr(),
+                              int(top), _stream()), "norm_add")
 
 
 def softcap(x: torch.Tensor, rows: int, cap: float) -> None:
@@ -1115,6 +1138,25 @@ def moe_plan(ids: torch.Tensor, slots: int, experts: int, sorted_slots: torch.Te
         raise ValueError("moe_plan: buffers too small")
     _check(_fn("bw_moe_plan")(ids.data_ptr(), slots, experts, sorted_slots.data_ptr(), place.data_ptr(), tiles.data_ptr(),
                               meta.data_ptr(), _stream()), "moe_plan")
+
+
+def moe_route_plan(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int, ids: torch.Tensor, wts: torch.Tensor,
+                   sorted_slots: torch.Tensor, place: torch.Tensor, tiles: torch.Tensor, meta: torch.Tensor) -> None:
+    """``moe_route`` followed by ``moe_plan`` over the rows' choices; steps of up to 16 rows do both in one launch."""
+    _need(logits, torch.float32, "logits")
+    _need(wts, torch.float32, "wts")
+    for t, what in ((ids, "ids"), (sorted_slots, "sorted"), (place, "place"), (tiles, "tiles"), (meta, "meta")):
+        _need(t, torch.int32, what)
+    experts, slots = logits.shape[1], rows * top
+    if logits.shape[0] < rows or min(ids.numel(), wts.numel(), sorted_slots.numel(), place.numel()) < slots:
+        raise ValueError("moe_route_plan: buffers shorter than the rows")
+    if experts % groups or not 1 <= keep <= groups or not 1 <= top <= keep * (experts // groups):
+        raise ValueError("moe_route_plan: groups, keep and top do not fit the experts")
+    if tiles.numel() < 4 * moe_max_tiles(slots, experts) or meta.numel() < 1:
+        raise ValueError("moe_route_plan: the plan's tables are too small")
+    _check(_fn("bw_moe_route_plan")(logits.data_ptr(), logits.stride(0), rows, experts, top, groups, keep, ids.data_ptr(), wts.data_ptr(),
+                                    sorted_slots.data_ptr(), place.data_ptr(), tiles.data_ptr(), meta.data_ptr(), _stream()),
+           "moe_route_plan")
 
 
 def moe_experts(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_slots: torch.Tensor, tiles: torch.Tensor,

@@ -264,6 +264,12 @@ class FeedForward(Part):
         out[:ctx.rows].zero_()
         self.forward(ctx, h, out)
 
+    def forward_add_normed(self, ctx, h, norm, x, rounded=None) -> bool:
+        """Optional: x += norm(feed_forward(h)) with the norm riding in the feed-forward's last kernel (``rounded`` as in
+        ``Norm.add_normed``).  Return False (and do nothing) if this part or this norm cannot; the block then calls
+        ``forward_out`` and the norm one after the other.  The result must be the same bits."""
+        return False
+
 
 class Block(Part):
     """The arrangement of a layer's parts around the residual stream.

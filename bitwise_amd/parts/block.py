@@ -98,5 +98,12 @@ class PostNormBlock(Block):
         self.mixer.forward_out(ctx, call, self._input(ctx, x), y)
         self._add(ctx, self.mixer_norm, y, x)
         if self.feed_forward is not None:
-            self.feed_forward.forward_out(ctx, self._input(ctx, x), y)
-            self._add(ctx, self.ffn_norm, y, x)
+            h = self._input(ctx, x)
+            notes = getattr(ctx, "forward_notes", None)
+            rounded = ctx.ws.buffer("stream_rounded", x.shape[1], torch.bfloat16) if (self.rt.bf16 and notes is not None) else None
+            if self.feed_forward.forward_add_normed(ctx, h, self.ffn_norm, x, rounded):
+                if rounded is not None:
+                    notes["stream_rounded"] = x
+            else:
+                self.feed_forward.forward_out(ctx, h, y)
+                self._add(ctx, self.ffn_norm, y, x)

@@ -77,7 +77,7 @@ class RoutedExperts(FeedForward):
         touched = self.experts * (1.0 - (1.0 - self.top / self.experts) ** max(int(rows), 1))
         return self.router.nbytes() + int(touched * per)
 
-    def _run(self, ctx, h, target, add: bool) -> None:
+    def _run(self, ctx, h, target, add: bool, norm=None, rounded=None) -> None:
         rt, ws, rows = self.rt, ctx.ws, ctx.rows
         slots = rows * self.top
         most = ws.max_rows * self.top
@@ -85,13 +85,12 @@ class RoutedExperts(FeedForward):
         self.router.store(ws, h, logits, rows)
         ids = ws.buffer("moe_ids", self.top, torch.int32)
         wts = ws.buffer("moe_wts", self.top, torch.float32)
-        ops.moe_route(logits, rows, self.top, self.groups, self.keep, ids, wts)
         sorted_slots = ws.buffer("moe_sorted", most, torch.int32, rows=1)
         place = ws.buffer("moe_place", most, torch.int32, rows=1)
         # (room for the plan of any step: tiles hold 16 slots or more, and every expert may end with a partly filled one)
         tiles = ws.buffer("moe_tiles", 4 * (most // 16 + self.experts), torch.int32, rows=1)
         meta = ws.buffer("moe_meta", 4, torch.int32, rows=1)
-        ops.moe_plan(ids, slots, self.experts, sorted_slots, place, tiles, meta)
+        ops.moe_route_plan(logits, rows, self.top, self.groups, self.keep, ids, wts, sorted_slots, place, tiles, meta)
         if self.mfma:
             x, act_dtype = h, torch.bfloat16
         else:
@@ -104,10 +103,23 @@ class RoutedExperts(FeedForward):
                         round_out=rt.bf16 and not self.mfma)
         y = ws.buffer("moe_y", self.width, torch.float32, rows=most)
         ops.moe_experts(act, self.down, y, sorted_slots, tiles, meta, slots, self.top, False)
-        ops.moe_combine(y, place, wts, self.top, target, rows, add)
+        if norm is not None:
+            # the rows' weighted sums are formed by the kernel that norms them and adds them into the stream
+            ops.norm_add(y, norm.weight, target, rows, norm.eps, rounded, combine=(place, wts, self.top))
+        else:
+            ops.moe_combine(y, place, wts, self.top, target, rows, add)
 
     def forward(self, ctx, h, residual) -> None:
         self._run(ctx, h, residual, True)
 
     def forward_out(self, ctx, h, out) -> None:
         self._run(ctx, h, out, False)
+
+    def forward_add_normed(self, ctx, h, norm, x, rounded=None) -> bool:
+        from .norm import RMSNorm
+        # (few rows: a launch that sums the choices over many workgroups and the norm's own launch are faster than one
+        # workgroup a row doing both; the bits are the same either way)
+        if type(norm) is not RMSNorm or ctx.rows <= 16:
+            return False
+        self._run(ctx, h, x, True, norm=norm, rounded=rounded)
+        return True

@@ -62,7 +62,11 @@ class RealGatedLRU(Mixer):
         wy, wx = tensors["y"], tensors["x"]
         if wy.dtype != wx.dtype:
             raise ValueError("the projections of one mixer must be stored in one dtype to be stacked")
-        self.proj = Linear(torch.cat([wy, wx], dim=0), self.rt, bias=torch.cat([tensors["y.b"].float(), tensors["x.b"].float()]))
+        self.proj = Linear(torch.cat([wy, wx], dim=0), self.rt)
+        # the projections' biases are added where their sums are first read: the convolution's inputs and the gate
+        # branch's activation (one 32-bit addition behind the product's sum either way)
+        self.y_bias = tensors["y.b"].to(dev).float().contiguous()
+        self.x_bias = tensors["x.b"].to(dev).float().contiguous()
         self.o = Linear(tensors["o"], self.rt)
         self.conv_w = tensors["conv"].to(dev).float().contiguous()
         self.conv_b = tensors["conv.b"].to(dev).float().contiguous()
@@ -76,7 +80,7 @@ class RealGatedLRU(Mixer):
         self.decay = (-self.decay_scale * torch.nn.functional.softplus(lam)).to(torch.float32).to(dev).contiguous()
 
     def weight_bytes(self) -> int:
-        small = (self.conv_w.numel() + self.conv_b.numel() + self.gate_w.numel() + 3 * self.inner) * 4
+        small = (self.conv_w.numel() + self.conv_b.numel() + self.gate_w.numel() + 5 * self.inner) * 4
         return self.proj.nbytes() + self.o.nbytes() + small
 
     def state_spec(self) -> StateSpec:
@@ -88,12 +92,12 @@ class RealGatedLRU(Mixer):
         self.proj.store(ws, h, proj, rows)
         u = ws.buffer("rglru_u", R, torch.float32)
         ops.causal_conv(proj[:, R:], self.conv_w, self.conv_b, call.state, ctx.seq_rows, ctx.slots, ctx.positions, ctx.nseq,
-                        max_seq_rows(ctx), u)
+                        max_seq_rows(ctx), u, in_bias=self.x_bias)
         gates = ws.buffer("rglru_gates", 2 * R, torch.float32)
         ops.headwise_linear(u, 0, self.bs, self.gate_w, gates, 0, 2 * self.bs, rows)
         act = ws.buffer("rglru_out", R, self.rt.act_dtype)
         ops.rglru_scan(proj, u, gates, self.ra_b, self.ri_b, self.decay, call.state[:, (self.taps - 1) * R:], act,
-                       ctx.seq_rows, ctx.slots, ctx.positions, ctx.nseq, rows, R, self.bs)
+                       ctx.seq_rows, ctx.slots, ctx.positions, ctx.nseq, rows, R, self.bs, y_bias=self.y_bias)
         if add:
             self.o.add_into(ws, act, target, rows)
         else:
